@@ -91,14 +91,16 @@ class HybridCache:
 
     * ``attention``:        (k [slots, G*d], v [slots, G*d])   token-major rows, slot =
                             block * block_size + offset; k holds the normed keys, v the raw ones
-    * ``latent_attention``: (c [slots, kv_rank + rot_dim],)     normed latent | rotated key
-    * ``hgrn2``:            (state [state_slots, H, d, dv] fp32,)  one slot per live sequence
+    * ``latent_attention``: (c [slots, kv_rank + rot_dim],)     normed latent | rotated key; a
+                            layer with ``kv_from`` gets that layer's tensor (it writes nothing)
+    * ``hgrn2``, ``gla``:   (state [state_slots, H, d, dv] fp32,)  one slot per live sequence
     * ``talk_attention``:   (k [slots, G*d], v [slots, G*dv])   normed keys and values; a layer
                             with ``kv_from`` gets the tensors of that layer's run (it writes
                             nothing)
 
     ``shift_states[run]`` is [state_slots, D] fp32 for a layer with token shift (the previous
-    token's mixer input), else None.
+    token's mixer input), else None. ``prev_token`` is int32 [state_slots] for a design whose
+    embedding reads the previous token (hashed bigrams), else None.
 
     Rows are zero-initialised once (padding rows of captured decode steps read row 0). A state
     slot is not cleared on reuse: a sequence's first portion starts from zero by position."""
@@ -113,12 +115,18 @@ class HybridCache:
         rows = num_blocks * block_size
         self.entries = []
         self.shift_states = []
+        self.prev_token = (torch.zeros(state_slots, dtype=torch.int32, device=device)
+                           if cfg.bigram else None)
         run_of = {}                       # layer -> its (last) run, for layers that lend their cache
         for ri, (li, _, _) in enumerate(cfg.layer_runs()):
             s = cfg.layer_specs[li]
             self.shift_states.append(
                 torch.zeros(state_slots, cfg.hidden_size, dtype=torch.float32, device=device)
                 if s.shift else None)
+            if s.kind == "latent_attention" and s.kv_from >= 0:
+                self.entries.append(self.entries[run_of[s.kv_from]])
+                run_of[li] = ri
+                continue
             if s.kind == "talk_attention":
                 if s.kv_from >= 0:
                     e = self.entries[run_of[s.kv_from]]

@@ -23,13 +23,22 @@ class LayerSpec:
     [dim, vdim] state per head), ``latent_attention`` (keys / values expanded from a cached
     low-rank latent plus one shared rotated key) and ``talk_attention`` (biased q / k / v
     projections, unit-RMS queries and keys, scores mixed across heads before the softmax,
-    attention inside blocks of ``chunk`` positions, optionally the cache of layer ``kv_from``).
+    attention inside blocks of ``chunk`` positions, optionally the cache of layer ``kv_from``)
+    and ``gla`` (gated linear attention: a [dim, vdim] state per head with independent keys and
+    a per-channel decay sigmoid(z)^(1/tau), z from a low-rank projection of width ``decay_rank``;
+    per-head RMS norm, SiLU output gate). ``latent_attention`` options: ``q_rank`` > 0 sends
+    the queries through an RMS-normed latent of that width, ``head_gate`` multiplies each
+    head's output by one sigmoid gate, ``rot_half`` pairs rotated dimension i with i +
+    rot_dims/2 instead of (2i, 2i+1), and ``kv_from`` reads another layer's cached latent.
 
     feed-forward kinds (``ff_kind``): ``gated_gelu`` (down(gelu(gate) * up)), ``gelu``
     (down(gelu(up))) and ``moe`` (``experts`` gated-SiLU experts of width ``ff`` plus
     ``identity`` pass-through experts, ``top`` per token chosen by softmax score + a learned
     correction and weighted by the un-renormalised score, and a shared expert of width
-    ``shared_ff`` behind a per-token sigmoid gate)."""
+    ``shared_ff`` behind a per-token sigmoid gate) and ``gated_silu`` (down(silu(gate) * up)).
+    A mixture with ``router`` = ``logit_topk`` picks the ``top`` largest biased logits and
+    weighs them by the softmax over the chosen ones; ``expert_act`` = ``gelu_erf`` makes the
+    experts (and the shared one, then ungated) down(gelu(up)) with the exact GELU."""
     kind: str
     heads: int
     dim: int
@@ -50,19 +59,26 @@ class LayerSpec:
     identity: int = 0
     top: int = 0
     shared_ff: int = 0
+    router: str = "score"     # "score" (softmax score + correction) | "logit_topk"
+    expert_act: str = "silu_mul"   # "silu_mul" (gated) | "gelu_erf" (ungated)
+    q_rank: int = 0           # latent attention: width of the query latent (0: none)
+    head_gate: bool = False   # latent attention: one sigmoid output gate per head
+    rot_half: bool = False    # rotation pairs (i, i + rot_dims/2) instead of (2i, 2i+1)
+    tau: float = 1.0          # gla: the decay is sigmoid(z)^(1/tau)
+    decay_rank: int = 0       # gla: inner width of the decay's two-step projection
 
     @property
     def has_state(self) -> bool:
         """The layer keeps something per sequence besides cache rows: a recurrent state, or
         the previous token's mixer input."""
-        return self.kind == "hgrn2" or self.shift
+        return self.kind in ("hgrn2", "gla") or self.shift
 
 
 @dataclass(frozen=True)
 class ModelConfig:
     name: str
     arch: str                 # "llama" (llama / mixtral family), "gpt2", or a hybrid
-                              # (layer-list) design: "buborax", "pulunex"
+                              # (layer-list) design: "buborax", "pulunex", "risutar"
     hidden_size: int
     num_layers: int
     num_heads: int
@@ -91,6 +107,14 @@ class ModelConfig:
     logit_scale: float = 1.0      # the LM head's output is multiplied by this
     learned_pos: bool = False     # a learned vector per position is added to the embedding
     scalar_norm: bool = False     # every norm's weight is one number (checkpoint layout)
+    # post-norm layers (arch "risutar"): x = LayerNorm(postln_alpha * x + sublayer(x)) with
+    # weight and bias, the sublayers reading x itself; 0 = pre-norm residual layers
+    postln_alpha: float = 0.0
+    # hashed bigram embedding (buckets, mul_prev, mul_cur): row (prev * mul_prev + cur *
+    # mul_cur) mod buckets of a second table is added, row ``buckets`` for a first token
+    bigram: tuple = ()
+    # per-layer token input: width of each layer's slice of a second embedding table
+    side_dim: int = 0
 
     @property
     def is_hybrid(self) -> bool:
@@ -113,7 +137,7 @@ class ModelConfig:
     def has_state(self) -> bool:
         """True when some layer keeps a recurrent state per sequence (state slots; such a
         model's prefix cannot be taken from cached KV blocks alone)."""
-        return any(s.has_state for s in self.layer_specs)
+        return bool(self.bigram) or any(s.has_state for s in self.layer_specs)
 
     @property
     def is_moe(self) -> bool:
@@ -176,7 +200,7 @@ class ModelConfig:
         if s.kind == "attention":
             return 2 * s.kv_heads * s.dim           # normed keys + raw keys (the values)
         if s.kind == "latent_attention":
-            return s.kv_rank + s.rot_dim
+            return 0 if s.kv_from >= 0 else s.kv_rank + s.rot_dim
         if s.kind == "talk_attention":
             return 0 if s.kv_from >= 0 else s.kv_heads * (s.dim + s.vdim)
         return 0
@@ -193,6 +217,8 @@ class ModelConfig:
                                       for s in kw["layer_specs"])
         if "loop" in kw:
             kw["loop"] = tuple(kw["loop"] or ())
+        if "bigram" in kw:
+            kw["bigram"] = tuple(kw["bigram"] or ())
         if "rope_scaling" in kw:         # JSON turned the pairs into lists
             kw["rope_scaling"] = tuple(tuple(p) for p in (kw["rope_scaling"] or ()))
         return cls(**kw)
@@ -282,9 +308,32 @@ PULUNEX_TINY = hybrid_config(
     layer_specs=(_pulunex_layer("gelu"), _pulunex_layer("moe"), _pulunex_layer("moe", kv_from=1)),
     norm_eps=1e-6, embed_scale=8.0, logit_scale=0.5, learned_pos=True, scalar_norm=True)
 
+def _risutar_moe(**kw) -> dict:
+    return dict(ff_kind="moe", router="logit_topk", expert_act="gelu_erf", **kw)
+
+
+_RISUTAR_LATENT = dict(heads=3, kv_heads=1, dim=32, vdim=40, scale=0.14, rot_dim=16, kv_rank=48,
+                       rot_dims=16, rot_base=5000.0, q_rank=40, head_gate=True, rot_half=True,
+                       window=1 << 30)
+
+# Risutar at test size: post-norm layers with bias, hashed bigram embedding, per-layer token
+# input, gated linear attention, latent attention with a query latent (one layer on another's
+# cache), dense and routed feed-forwards, a layer without feed-forward
+RISUTAR_TINY = hybrid_config(
+    "risutar-tiny", width=128, vocab=384, arch="risutar",
+    layer_specs=(
+        LayerSpec("latent_attention", **_RISUTAR_LATENT, ff=192, ff_kind="gated_silu"),
+        LayerSpec("gla", heads=2, dim=24, vdim=32, tau=8.0, decay_rank=8,
+                  **_risutar_moe(ff=48, experts=5, top=2, shared_ff=64)),
+        LayerSpec("latent_attention", **_RISUTAR_LATENT, kv_from=0,
+                  **_risutar_moe(ff=64, experts=4, top=1)),
+        LayerSpec("gla", heads=4, dim=16, vdim=16, tau=4.0, decay_rank=4, ff=0)),
+    norm_eps=1e-5, postln_alpha=2.0, bigram=(251, 31, 5), side_dim=8)
+
 _REGISTRY = {c.name: c for c in
              (GPT2, LLAMA3_8B, LLAMA3_70B, MIXTRAL_8X7B, LLAMA_TINY, LLAMA_TINY128,
-              LLAMA_TINY8, MIXTRAL_TINY, MIXTRAL_TINY8E, GPT2_TINY, BUBORAX_TINY, PULUNEX_TINY)}
+              LLAMA_TINY8, MIXTRAL_TINY, MIXTRAL_TINY8E, GPT2_TINY, BUBORAX_TINY, PULUNEX_TINY,
+              RISUTAR_TINY)}
 
 _ALIASES = {
     "openai-community/gpt2": "gpt2",

@@ -25,7 +25,8 @@ from typing import Dict, Iterable, Iterator, Optional, Tuple
 import torch
 
 from .configs import ModelConfig
-from .weights import from_buborax_state_dict, from_hf_state_dict, from_pulunex_state_dict
+from .weights import (from_buborax_state_dict, from_hf_state_dict, from_pulunex_state_dict,
+                      from_risutar_state_dict)
 
 
 def is_hf_dir(d) -> bool:
@@ -58,7 +59,7 @@ def find_hf_dir(root: str, name: str) -> Optional[Path]:
     return None
 
 
-NATIVE_ARCHS = ("Buborax", "Pulunex")
+NATIVE_ARCHS = ("Buborax", "Pulunex", "Risutar")
 
 
 def buborax_config(c: dict, name: Optional[str] = None) -> ModelConfig:
@@ -160,13 +161,77 @@ def pulunex_config(c: dict, name: Optional[str] = None) -> ModelConfig:
                          scalar_norm=True)
 
 
+def risutar_config(c: dict, name: Optional[str] = None) -> ModelConfig:
+    """A Risutar ``config.json``: ``width``, ``vocab``, ``norm`` {eps}, ``postln_alpha``,
+    ``embedding`` {bigram {buckets, mul_prev, mul_cur}} (optional), ``token_side`` {dim}
+    (optional) and ``layers``, a list of {type, mixer, mlp}: type ``gla`` with mixer {heads, dim,
+    vdim, tau} or ``latent_attention`` with mixer {heads, dim, rot_dim, vdim, kv_rank, q_rank,
+    scale, rot {base, dims}, kv_from}; mlp null, {kind: dense, ff} or {kind: moe, expert {ff},
+    router {experts, top}, shared {ff}}. Sizes a config does not carry (the decay's inner
+    width) come from the tensors' shapes at load time."""
+    from .configs import LayerSpec, hybrid_config
+    specs = []
+    for i, L in enumerate(c["layers"]):
+        mx, kind = L["mixer"], L["type"]
+        ff = dict(ff=0)
+        mlp = L.get("mlp")
+        if mlp:
+            fk = mlp.get("kind", "dense")
+            if fk == "dense":
+                ff = dict(ff=int(mlp["ff"]), ff_kind="gated_silu")
+            elif fk == "moe":
+                r = mlp["router"]
+                ff = dict(ff=int(mlp["expert"]["ff"]), ff_kind="moe", router="logit_topk",
+                          expert_act="gelu_erf", experts=int(r["experts"]), top=int(r["top"]),
+                          shared_ff=int((mlp.get("shared") or {}).get("ff") or 0))
+                if not 1 <= ff["top"] <= ff["experts"]:
+                    raise ValueError(f"layer {i}: router.top {ff['top']} of {ff['experts']} experts")
+            else:
+                raise ValueError(f"unsupported feed-forward kind '{fk}'")
+        H, d = int(mx["heads"]), int(mx["dim"])
+        if kind == "gla":
+            specs.append(LayerSpec("gla", heads=H, dim=d, vdim=int(mx.get("vdim", d)),
+                                   tau=float(mx.get("tau", 1.0)),
+                                   decay_rank=int(mx.get("decay_rank") or 0), **ff))
+        elif kind == "latent_attention":
+            rot = mx.get("rot") or {}
+            dr = int(mx["rot_dim"])
+            src = mx.get("kv_from")
+            src = -1 if src is None else int(src)
+            r = int(mx["kv_rank"])
+            if src >= 0:
+                o = specs[src] if src < i else None
+                if (o is None or o.kind != "latent_attention" or o.kv_from >= 0
+                        or (o.kv_rank, o.rot_dim) != (r, dr)):
+                    raise ValueError(f"layer {i}: kv_from {src} must name an earlier latent-"
+                                     "attention layer with a projection of its own and the "
+                                     "same latent and rotated sizes")
+            specs.append(LayerSpec("latent_attention", heads=H, kv_heads=1, dim=d,
+                                   vdim=int(mx["vdim"]), window=1 << 30,
+                                   scale=float(mx.get("scale", (d + dr) ** -0.5)), rot_dim=dr,
+                                   kv_rank=r, rot_dims=int(rot.get("dims", dr)),
+                                   rot_base=float(rot.get("base", 10000.0)),
+                                   q_rank=int(mx.get("q_rank") or 0), head_gate=True,
+                                   rot_half=True, kv_from=src, **ff))
+        else:
+            raise ValueError(f"unsupported mixer type '{kind}'")
+    bg = (c.get("embedding") or {}).get("bigram")
+    bigram = (int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"])) if bg else ()
+    return hybrid_config(name or c.get("_name_or_path") or "risutar", int(c["width"]),
+                         int(c["vocab"]), specs, norm_eps=float((c.get("norm") or {}).get("eps", 1e-5)),
+                         arch="risutar", postln_alpha=float(c.get("postln_alpha", 1.0)),
+                         bigram=bigram, side_dim=int((c.get("token_side") or {}).get("dim") or 0))
+
+
 def config_from_hf(c: dict, name: Optional[str] = None) -> ModelConfig:
     """Map a ``config.json``: HF llama / mistral / mixtral / gpt2 model types, or one of the
-    native layer-list designs (``architecture``: Buborax, Pulunex)."""
+    native layer-list designs (``architecture``: Buborax, Pulunex, Risutar)."""
     if c.get("architecture") == "Buborax":
         return buborax_config(c, name)
     if c.get("architecture") == "Pulunex":
         return pulunex_config(c, name)
+    if c.get("architecture") == "Risutar":
+        return risutar_config(c, name)
     mt = c.get("model_type", "")
     name = name or c.get("_name_or_path") or mt
     if mt == "gpt2":
@@ -278,6 +343,8 @@ def load_hf_dir(d, device="cpu", dtype=torch.bfloat16, name: Optional[str] = Non
     try:
         if cfg.arch == "pulunex":
             params = from_pulunex_state_dict(cfg, sd, dtype=dtype)
+        elif cfg.arch == "risutar":
+            cfg, params = from_risutar_state_dict(cfg, sd, dtype=dtype)
         elif cfg.is_hybrid:
             params = from_buborax_state_dict(cfg, sd, dtype=dtype)
         else:

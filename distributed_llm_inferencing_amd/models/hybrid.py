@@ -1,11 +1,20 @@
-"""Hybrid decoder (archs ``buborax``, ``pulunex``): a layer list that mixes windowed attention,
-latent attention, a gated linear recurrence and block attention with head-mixed scores; dense,
-gated and routed feed-forwards; a shared-weight loop, grouped RMS norms, token shift and an
-fp32 residual stream — served by the same engine, scheduler, block manager and runner as the
-transformer families.
+"""Hybrid decoder (archs ``buborax``, ``pulunex``, ``risutar``): a layer list that mixes
+windowed attention, latent attention, gated linear recurrences (HGRN2, gated linear attention)
+and block attention with head-mixed scores; dense, gated and routed feed-forwards; a
+shared-weight loop, grouped RMS norms, token shift and an fp32 residual stream — served by the
+same engine, scheduler, block manager and runner as the transformer families.
 
     embed (fp32) -> per layer run: x += m * mixer(gnorm(x)); x += m * ff(gnorm(x))
                  -> gnorm -> LM head (fp32 logits) -> sampler
+
+Post-norm designs (``cfg.postln_alpha``; ``risutar``) run
+
+    embed + hashed bigram (fp32) -> per layer: x = LN(a x + mixer(x)); x = LN(a x + ff(x));
+                 x += rmsnorm(side_proj(gelu(side_gate x) * side_embed[token]))
+                 -> LN -> LM head
+
+with layer norms that carry weight and bias, the sublayers reading x itself (its rounding to
+the storage dtype feeds the GEMMs; the stream, the norms and the sums stay fp32).
 
 * Layers [start, stop) of the loop run ``times`` times with the same weights; a pass starts
   with x = W_in [x ; x0] + step[pass] (x0 = the embedding output). Every run owns its cache or
@@ -48,6 +57,7 @@ class HybridLM(TransformerLM):
         for spec, lp in zip(cfg.layer_specs, self.layers):
             derive_constants(spec, lp, self.device)
         self._cu: Dict[int, torch.Tensor] = {}
+        self._rows: Dict[int, torch.Tensor] = {}
         # debugging aid: when a list, forward_layers appends the residual after every run
         self.layer_trace: Optional[List[torch.Tensor]] = None
 
@@ -59,6 +69,7 @@ class HybridLM(TransformerLM):
         for spec, lp in zip(self.cfg.layer_specs, self.layers):
             derive_constants(spec, lp, self.device)
         self._cu.clear()
+        self._rows.clear()
         return self
 
     # ------------------------------------------------------------------ step metadata
@@ -77,15 +88,54 @@ class HybridLM(TransformerLM):
         return StepView(cu, mx, b.positions, b.slot_mapping, b.block_tables, block_size,
                         b.state_slots)
 
+    def _all_rows(self, n: int) -> torch.Tensor:
+        r = self._rows.get(n)
+        if r is None:
+            r = self._rows[n] = torch.arange(n, dtype=torch.int64, device=self.device)
+        return r
+
     # ------------------------------------------------------------------ forward
-    def embed(self, b: DeviceBatch) -> torch.Tensor:
+    def embed(self, b: DeviceBatch, kv_caches=None) -> torch.Tensor:
         cfg, p = self.cfg, self.params
+        if cfg.postln_alpha:
+            # (fp32 stream, its storage-dtype rounding): the first layer's sublayers read both
+            prev, bg = None, cfg.bigram or (0, 0, 0)
+            if cfg.bigram:
+                step = self._step_view(b, kv_caches.block_size)
+                prev = H.prev_tokens(b.input_ids, kv_caches.prev_token, step.state_slots,
+                                     step.cu_seqlens, step.max_seqlen, step.positions)
+            return H.embedding_bigram(b.input_ids, prev, p["embed"], p.get("bigram"), *bg)
         return H.embedding_f32(b.input_ids, p["embed"], scale=cfg.embed_scale,
                                pos_table=p.get("pos_embed") if cfg.learned_pos else None,
                                positions=b.positions)[0]
 
+    def _postnorm_layers(self, xs, b: DeviceBatch, kv_caches) -> torch.Tensor:
+        """Post-norm layers: every sublayer reads the stream itself and the norm follows the
+        sum. ``xs`` = (fp32 stream, its storage-dtype copy)."""
+        cfg, p = self.cfg, self.params
+        eps, a = cfg.norm_eps, cfg.postln_alpha
+        step = self._step_view(b, kv_caches.block_size)
+        x, xb = xs
+        for li, (spec, lp) in enumerate(zip(cfg.layer_specs, self.layers)):
+            y = MIXERS[spec.kind](spec, lp, xb, step, kv_caches.entries[li], eps)
+            xb = H.postnorm(x, y, lp["norm1"], lp["norm1_b"], eps, keep=a)
+            if spec.ff:
+                y = FEED_FORWARDS[spec.ff_kind](spec, lp, xb)
+                xb = H.postnorm(x, y, lp["norm2"], lp["norm2_b"], eps, keep=a)
+            elif "norm2" in lp:
+                xb = H.postnorm(x, None, lp["norm2"], lp["norm2_b"], eps, keep=a)
+            if cfg.side_dim:            # per-layer token input
+                g = H.side_gate(H.linear_any(xb, lp["side_gate"]), b.input_ids, p["side_embed"],
+                                li * cfg.side_dim)
+                xb = H.add_rmsnormed(x, H.linear_any(g, lp["side_proj"]), lp["side_norm"], eps)
+            if self.layer_trace is not None:
+                self.layer_trace.append(x.clone())
+        return x
+
     def forward_layers(self, x: torch.Tensor, b: DeviceBatch, kv_caches) -> torch.Tensor:
         cfg, p = self.cfg, self.params
+        if cfg.postln_alpha:
+            return self._postnorm_layers(x, b, kv_caches)
         eps, groups, m = cfg.norm_eps, cfg.norm_groups, cfg.residual_mult
         step = self._step_view(b, kv_caches.block_size)
         entries = kv_caches.entries
@@ -126,6 +176,13 @@ class HybridLM(TransformerLM):
         elif b.is_prefill:
             rows = b.last_token_idx
         else:
+            rows = None
+        if cfg.postln_alpha:
+            if rows is None:
+                rows = self._all_rows(hidden.shape[0])
+            return H.postnorm(hidden, None, p["final_norm"], p["final_norm_b"], cfg.norm_eps,
+                              rows_idx=rows)
+        if rows is None:
             return H.resadd_groupnorm(hidden, None, p["final_norm"], cfg.norm_groups,
                                       cfg.norm_eps, gain=cfg.logit_scale)
         # the logit scale rides on the final norm's output: the head is linear
@@ -139,7 +196,7 @@ class HybridLM(TransformerLM):
                 return_logits: bool = False):
         """Sampled int32 tokens [S] (and the logits when asked). With ``b.logit_rows`` the
         logits of exactly those rows are returned and nothing is sampled."""
-        x = self.forward_layers(self.embed(b), b, kv_caches)
+        x = self.forward_layers(self.embed(b, kv_caches), b, kv_caches)
         lg = self.logits(x, b)
         if b.logit_rows is not None:
             return lg

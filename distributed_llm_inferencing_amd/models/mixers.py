@@ -42,12 +42,15 @@ def derive_constants(spec: LayerSpec, lp: dict, device) -> None:
         lp["slopes"] = torch.pow(2.0, -8.0 * h / spec.heads).float().to(device)
         lp["talk"] = lp["talk"].float().contiguous()
     elif spec.kind == "latent_attention":
+        # float64: the angle position * frequency is formed in double and rounded once
         i = torch.arange(spec.rot_dims // 2, dtype=torch.float64)
-        lp["inv_freq"] = torch.pow(spec.rot_base, -2.0 * i / max(1, spec.rot_dims)).float().to(device)
+        lp["inv_freq"] = torch.pow(spec.rot_base, -2.0 * i / max(1, spec.rot_dims)).to(device)
     elif spec.kind == "talk_attention":
         lp["talk"] = lp["talk"].float().contiguous()
-    if spec.ff_kind == "moe" and spec.ff:
+    if spec.ff_kind == "moe" and spec.ff and spec.router == "score":
         lp["correction"] = lp["correction"].float().contiguous()
+    if spec.ff_kind == "moe" and spec.ff and spec.router == "logit_topk":
+        lp["router_b"] = lp["router_b"].float().contiguous()
 
 
 def attention_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, eps: float):
@@ -86,16 +89,51 @@ def latent_attention_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, 
     Hh, d, dr, dv, r = spec.heads, spec.dim, spec.rot_dim, spec.vdim, spec.kv_rank
     (c,) = cache
     T = h.shape[0]
-    proj = H.linear_any(h, lp["w_in"])                       # fp32 [T, q heads | ckv | k_rot]
-    q_nope, q_full = H.mla_prepare(proj, lp["c_norm"], eps, Hh, d, dr, r, spec.rot_dims,
-                                   lp["inv_freq"], step.positions, step.slot_mapping, c)
+    proj = H.linear_any(h, lp["w_in"])
+    gates = None
+    if spec.q_rank or spec.head_gate or spec.kv_from >= 0 or spec.rot_half:
+        # fp32 [T, query latent (or q heads) | ckv | k_rot (own cache only) | head gates]
+        nq = spec.q_rank or Hh * (d + dr)
+        qproj = proj[:, :nq]
+        if spec.q_rank:                     # queries through an RMS-normed latent
+            qproj = H.linear_any(H.rmsnorm_cols(qproj, lp["q_norm"], eps), lp["w_uq"])
+        own = spec.kv_from < 0
+        kvproj = proj[:, nq:nq + r + dr] if own else None
+        if spec.head_gate:
+            g0 = nq + (r + dr if own else 0)
+            gates = proj[:, g0:g0 + Hh]
+        q_nope, q_full = H.latent_prepare(qproj, kvproj, lp.get("c_norm"), eps, Hh, d, dr, r,
+                                          spec.rot_dims, lp["inv_freq"], step.positions,
+                                          step.slot_mapping, c, h.dtype, spec.rot_half)
+    else:                                   # fp32 [T, q heads | ckv | k_rot]
+        q_nope, q_full = H.mla_prepare(proj, lp["c_norm"], eps, Hh, d, dr, r, spec.rot_dims,
+                                       lp["inv_freq"], step.positions, step.slot_mapping, c)
     H.head_linear(q_nope, lp["w_ukT"], q_full)               # q_full[:, h, :r] = W_uk,h^T q_h
     ol = H.window_attention(q_full.view(T, Hh * (r + dr)), c, c, r + dr, r, Hh, 1,
                             step.cu_seqlens, step.max_seqlen, step.positions,
                             step.block_tables, step.block_size, spec.window, spec.scale)
+    if gates is not None:                   # one sigmoid gate per head, on the fp32 expansion
+        o32 = torch.empty(T, Hh, dv, dtype=torch.float32, device=h.device)
+        H.head_linear(ol.view(T, Hh, r), lp["w_uv"], o32)
+        return H.linear_any(H.head_gate(o32, gates, h.dtype), lp["wo"])
     o = torch.empty(T, Hh, dv, dtype=h.dtype, device=h.device)
     H.head_linear(ol.view(T, Hh, r), lp["w_uv"], o)
     return H.linear_any(o.view(T, Hh * dv), lp["wo"])
+
+
+def gla_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, eps: float):
+    """Gated linear attention: independent keys, a per-channel decay sigmoid(z)^(1/tau) with z
+    from a two-step low-rank projection, per-head RMS norm of the read-out, SiLU output gate.
+    The projections run in the storage dtype; the decay, the state and the norm in fp32."""
+    (state,) = cache
+    Hh, d, dv = spec.heads, spec.dim, spec.vdim
+    proj = H.linear_any(h, lp["w_in"])          # fp32 [T, q | k | v | gate | decay-in]
+    a0 = 2 * Hh * (d + dv)
+    a1 = H.act_mul(proj[:, a0:], spec.decay_rank, h.dtype, "copy")
+    z = H.linear_any(a1, lp["w_a2"])
+    o = H.gla(proj, z, lp["a_b"], spec.tau, lp["o_norm"], eps, state, step.state_slots,
+              step.cu_seqlens, step.max_seqlen, step.positions, Hh, d, dv)
+    return H.linear_any(o, lp["wo"])
 
 
 def talk_attention_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, eps: float):
@@ -116,7 +154,8 @@ def talk_attention_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, ep
 
 
 MIXERS = {"attention": attention_mixer, "hgrn2": hgrn2_mixer,
-          "latent_attention": latent_attention_mixer, "talk_attention": talk_attention_mixer}
+          "latent_attention": latent_attention_mixer, "talk_attention": talk_attention_mixer,
+          "gla": gla_mixer}
 
 
 # ----------------------------------------------------------------------------- feed-forwards
@@ -132,7 +171,8 @@ def prepare_feed_forward(spec: LayerSpec, params: dict, pre: str) -> None:
     from ..ops.reference import interleave_gate_up
     w = params.get(pre + "w_down")
     if (not spec.ff or w is None or pre + "ff_tuned" in params or w.dtype != torch.bfloat16
-            or not w.is_cuda or spec.ff_kind not in ("gelu", "moe") or w.shape[-2] % 64
+            or not w.is_cuda or spec.ff_kind not in ("gelu", "moe") or spec.router != "score"
+            or w.shape[-2] % 64
             or spec.ff % 64 or spec.shared_ff % 64):
         return
     if spec.ff_kind == "gelu":
@@ -161,8 +201,19 @@ def gelu_ff(spec: LayerSpec, lp: dict, h):
     return H.linear_any(act, lp["w_down"])
 
 
+def gated_silu_ff(spec: LayerSpec, lp: dict, h):
+    act = H.act_mul(H.linear_any(h, lp["w_gu"]), spec.ff, h.dtype, "silu_mul")
+    return H.linear_any(act, lp["w_down"])
+
+
 def moe_ff(spec: LayerSpec, lp: dict, h):
-    """Routed gated-SiLU experts + identity experts + a gated shared expert, summed in fp32."""
+    """Routed gated-SiLU experts + identity experts + a gated shared expert, summed in fp32;
+    with ``router`` = ``logit_topk``: biased logits, softmax over the chosen, ungated exact-GELU
+    experts and an always-on shared expert."""
+    if spec.router == "logit_topk":
+        tw, ti = H.logit_router(h, lp["router"], lp["router_b"], spec.top)
+        shared = (lp["ws_up"], lp["ws_down"]) if spec.shared_ff else None
+        return H.moe_gelu_experts_f32(h, lp["w_up"], lp["w_down"], tw, ti, shared)
     ng = 1 if spec.shared_ff else 0
     tw, ti, gates = H.score_router(h, lp["router"], lp["correction"], spec.top, ng)
     if "ff_tuned" not in lp:
@@ -177,4 +228,5 @@ def moe_ff(spec: LayerSpec, lp: dict, h):
     return H.moe_finish(routed, tw, ti, h, lp["w_gu"].shape[0], ys, gates if ng else None)
 
 
-FEED_FORWARDS = {"gated_gelu": gated_gelu_ff, "gelu": gelu_ff, "moe": moe_ff}
+FEED_FORWARDS = {"gated_gelu": gated_gelu_ff, "gelu": gelu_ff, "moe": moe_ff,
+                 "gated_silu": gated_silu_ff}

@@ -45,7 +45,17 @@ def hybrid_layer_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
         gelu:           w_up [F, D], w_down [D, F]
         moe:            router [E + I (+ 1), D] (the last row is the shared expert's gate),
                         correction [E + I] fp32, w_gu [E, 2F, D] = gate | up per expert,
-                        w_down [E, D, F], shared expert ws_gu [2Fs, D], ws_down [D, Fs]"""
+                        w_down [E, D, F], shared expert ws_gu [2Fs, D], ws_down [D, Fs]
+        gated_silu:     w_gu [2F, D] = gate | up, w_down [D, F]
+        moe, router ``logit_topk`` with ``gelu_erf`` experts: router [E, D], router_b [E] fp32,
+                        w_up [E, F, D], w_down [E, D, F], shared ws_up [Fs, D], ws_down [D, Fs]
+      gla:              w_in [2*H*d + 2*H*dv + ra, D] = q | k | v | output gate | decay-in,
+                        w_a2 [H*d, ra], a_b [H*d], o_norm [dv], wo [D, H*dv]
+      latent_attention with ``q_rank`` / ``head_gate``: w_in [rq + (r + dr) + H, D] = query
+                        latent | compressed kv (absent with ``kv_from``) | head gates,
+                        q_norm [rq], w_uq [H*(d+dr), rq], then as above
+    Post-norm designs add the norms' biases norm1_b / norm2_b [D]; with a per-layer token input
+    of width s: side_gate [s, D], side_proj [D, s], side_norm [D]."""
     D = cfg.hidden_size
     s = cfg.layer_specs[i]
     p = f"layers.{i}."
@@ -58,16 +68,38 @@ def hybrid_layer_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
         out.update({p + "w_in": (2 * H * d + H * dv, D), p + "f_b": (H * d,),
                     p + "lower": (H * d,), p + "o_norm": (dv,), p + "wo": (D, H * dv)})
     elif s.kind == "latent_attention":
-        out.update({p + "w_in": (H * (d + s.rot_dim) + s.kv_rank + s.rot_dim, D),
-                    p + "c_norm": (s.kv_rank,), p + "w_ukT": (H, s.kv_rank, d),
+        nkv = 0 if s.kv_from >= 0 else s.kv_rank + s.rot_dim
+        nq = s.q_rank if s.q_rank else H * (d + s.rot_dim)
+        out.update({p + "w_in": (nq + nkv + (H if s.head_gate else 0), D),
+                    p + "w_ukT": (H, s.kv_rank, d),
                     p + "w_uv": (H, dv, s.kv_rank), p + "wo": (D, H * dv)})
+        if nkv:
+            out[p + "c_norm"] = (s.kv_rank,)
+        if s.q_rank:
+            out.update({p + "q_norm": (s.q_rank,), p + "w_uq": (H * (d + s.rot_dim), s.q_rank)})
+    elif s.kind == "gla":
+        ra = s.decay_rank
+        out.update({p + "w_in": (2 * H * d + 2 * H * dv + ra, D), p + "w_a2": (H * d, ra),
+                    p + "a_b": (H * d,), p + "o_norm": (dv,), p + "wo": (D, H * dv)})
     elif s.kind == "talk_attention":
         n_in = H * d + (0 if s.kv_from >= 0 else s.kv_heads * (d + dv))
         out.update({p + "shift": (D,), p + "w_in": (n_in, D), p + "b_in": (n_in,),
                     p + "talk": (H, H), p + "wo": (D, H * dv)})
     else:
         raise ValueError(f"unknown mixer kind '{s.kind}'")
-    if s.ff and s.ff_kind == "gated_gelu":
+    if cfg.postln_alpha:
+        out[p + "norm1_b"] = (D,)
+        if s.ff:
+            out[p + "norm2_b"] = (D,)
+    if cfg.side_dim:
+        out.update({p + "side_gate": (cfg.side_dim, D), p + "side_proj": (D, cfg.side_dim),
+                    p + "side_norm": (D,)})
+    if s.ff and s.ff_kind == "moe" and s.router == "logit_topk":
+        out.update({p + "norm2": (D,), p + "router": (s.experts, D), p + "router_b": (s.experts,),
+                    p + "w_up": (s.experts, s.ff, D), p + "w_down": (s.experts, D, s.ff)})
+        if s.shared_ff:
+            out.update({p + "ws_up": (s.shared_ff, D), p + "ws_down": (D, s.shared_ff)})
+    elif s.ff and s.ff_kind in ("gated_gelu", "gated_silu"):
         out.update({p + "norm2": (D,), p + "w_gu": (2 * s.ff, D), p + "w_down": (D, s.ff)})
     elif s.ff and s.ff_kind == "gelu":
         out.update({p + "norm2": (D,), p + "w_up": (s.ff, D), p + "w_down": (D, s.ff)})
@@ -113,6 +145,12 @@ def global_param_shapes(cfg: ModelConfig, first: bool, last: bool) -> Dict[str, 
             s.update({"loop_in": (d, 2 * d), "loop_step": (cfg.loop[2], d)})
         if cfg.learned_pos:
             s["pos_embed"] = (cfg.max_position, d)
+        if cfg.postln_alpha:
+            s["final_norm_b"] = (d,)
+        if cfg.bigram:
+            s["bigram"] = (cfg.bigram[0] + 1, d)
+        if cfg.side_dim:
+            s["side_embed"] = (v, len(cfg.layer_specs) * cfg.side_dim)
         return s
     if first or (last and cfg.tie_embeddings):
         s["embed"] = (v, d)
@@ -143,11 +181,12 @@ def stage_param_shapes(cfg: ModelConfig, layer_start: int, layer_end: int, first
 
 def _is_norm_weight(name: str) -> bool:
     return name.endswith(("attn_norm", "mlp_norm", "final_norm", "ln1_w", "ln2_w", "norm1",
-                          "norm2", "q_norm", "k_norm", "c_norm", "o_norm"))
+                          "norm2", "q_norm", "k_norm", "c_norm", "o_norm", "side_norm"))
 
 
 def _is_bias(name: str) -> bool:
-    return name.endswith(("ln1_b", "ln2_b", "bqkv", "bo", "b_fc", "b_proj", "final_norm_b"))
+    return name.endswith(("ln1_b", "ln2_b", "bqkv", "bo", "b_fc", "b_proj", "final_norm_b",
+                          "norm1_b", "norm2_b"))
 
 
 def random_init(shapes: Dict[str, tuple], device, dtype=torch.bfloat16, seed: int = 0,
@@ -159,7 +198,7 @@ def random_init(shapes: Dict[str, tuple], device, dtype=torch.bfloat16, seed: in
     hybrid = any(n.endswith(".norm1") for n in shapes)
     for name in sorted(shapes):
         shape = shapes[name]
-        if hybrid and not _is_norm_weight(name):
+        if hybrid and not _is_norm_weight(name) and not _is_bias(name):
             out[name] = _hybrid_init(name, shape, dev, dtype, seed)
         elif _is_norm_weight(name):
             out[name] = torch.ones(shape, dtype=dtype, device=dev)
@@ -186,6 +225,11 @@ def _hybrid_init(name: str, shape: tuple, dev, dtype, seed: int) -> torch.Tensor
         return t.to(dev, torch.float32)
     if name.endswith(".correction"):
         return (0.05 * torch.randn(shape, generator=g)).to(dev, torch.float32)
+    if name.endswith(".router_b"):
+        return (0.1 * torch.randn(shape, generator=g)).to(dev, torch.float32)
+    if name.endswith(".a_b"):
+        # decays sigmoid(z)^(1/tau) spread between fast and slow channels
+        return (1.0 + 2.0 * torch.randn(shape, generator=g)).to(dev, dtype)
     if name.endswith(".shift"):
         return torch.rand(shape, generator=g).to(dev, dtype)
     if name.endswith(".b_in"):
@@ -378,3 +422,66 @@ def from_pulunex_state_dict(cfg: ModelConfig, sd, dtype=torch.bfloat16) -> Dict[
             out[p + "ws_gu"] = cv(torch.cat([sd[f + "shared.gate"], sd[f + "shared.up"]], 0))
             out[p + "ws_down"] = cv(sd[f + "shared.down"])
     return out
+
+
+# ----------------------------------------------------------------------------- Risutar files
+def from_risutar_state_dict(cfg: ModelConfig, sd, dtype=torch.bfloat16):
+    """Convert a Risutar checkpoint (tensor names ``embed``, ``bigram``, ``side.embed``,
+    ``head``, ``final.norm`` (+ ``.b``), ``l<i>.norm1|norm2`` (+ ``.b``), ``l<i>.mix.*``,
+    ``l<i>.mlp.*``, ``l<i>.side.gate|proj|norm``; linear weights [out, in]) into the layout of
+    ``hybrid_layer_shapes``: projections that read the layer input are stacked, the experts are
+    stacked, W_uk is stored per head and transposed (the absorb projection). Returns (config,
+    tensors): widths the config file does not carry (the decay's inner width, the query
+    latent's) are taken from the tensors' shapes."""
+    from dataclasses import replace
+    cv = lambda t: t.detach().to(dtype).contiguous()  # noqa: E731
+    out = {"embed": cv(sd["embed"]), "lm_head": cv(sd["head"]),
+           "final_norm": cv(sd["final.norm"]), "final_norm_b": cv(sd["final.norm.b"])}
+    if cfg.bigram:
+        out["bigram"] = cv(sd["bigram"])
+    if cfg.side_dim:
+        out["side_embed"] = cv(sd["side.embed"])
+    specs = list(cfg.layer_specs)
+    for i, s in enumerate(specs):
+        a, p = f"l{i}.", f"layers.{i}."
+        m = a + "mix."
+        out[p + "norm1"], out[p + "norm1_b"] = cv(sd[a + "norm1"]), cv(sd[a + "norm1.b"])
+        H, d, dv = s.heads, s.dim, s.vdim
+        if s.kind == "gla":
+            a1 = sd[m + "a1"]
+            specs[i] = s = replace(s, decay_rank=int(a1.shape[0]))
+            out[p + "w_in"] = cv(torch.cat([sd[m + "q"], sd[m + "k"], sd[m + "v"], sd[m + "g"],
+                                            a1], 0))
+            out[p + "w_a2"], out[p + "a_b"] = cv(sd[m + "a2"]), cv(sd[m + "a2.b"])
+            out[p + "o_norm"] = cv(sd[m + "norm"])
+        else:
+            dq = sd[m + "dq"]
+            specs[i] = s = replace(s, q_rank=int(dq.shape[0]))
+            parts = [dq] + ([] if s.kv_from >= 0 else [sd[m + "dkv"]]) + [sd[m + "g"]]
+            out[p + "w_in"] = cv(torch.cat(parts, 0))
+            out[p + "q_norm"], out[p + "w_uq"] = cv(sd[m + "dq.norm"]), cv(sd[m + "uq"])
+            if s.kv_from < 0:
+                out[p + "c_norm"] = cv(sd[m + "dkv.norm"])
+            uk = sd[m + "uk"].detach().reshape(H, d, s.kv_rank)
+            out[p + "w_ukT"] = cv(uk.transpose(1, 2))
+            out[p + "w_uv"] = cv(sd[m + "uv"].detach().reshape(H, dv, s.kv_rank))
+        out[p + "wo"] = cv(sd[m + "o"])
+        if cfg.side_dim:
+            for n in ("gate", "proj", "norm"):
+                out[p + "side_" + n] = cv(sd[f"{a}side.{n}"])
+        if s.ff or a + "norm2" in sd:     # a second norm without a feed-forward still norms
+            out[p + "norm2"], out[p + "norm2_b"] = cv(sd[a + "norm2"]), cv(sd[a + "norm2.b"])
+        if not s.ff:
+            continue
+        f = a + "mlp."
+        if s.ff_kind == "gated_silu":
+            out[p + "w_gu"] = cv(torch.cat([sd[f + "gate"], sd[f + "up"]], 0))
+            out[p + "w_down"] = cv(sd[f + "down"])
+            continue
+        out[p + "router"] = cv(sd[f + "router"])
+        out[p + "router_b"] = sd[f + "router.b"].detach().float().contiguous()
+        out[p + "w_up"] = cv(torch.stack([sd[f"{f}e{e}.up"] for e in range(s.experts)]))
+        out[p + "w_down"] = cv(torch.stack([sd[f"{f}e{e}.down"] for e in range(s.experts)]))
+        if s.shared_ff:
+            out[p + "ws_up"], out[p + "ws_down"] = cv(sd[f + "shared.up"]), cv(sd[f + "shared.down"])
+    return replace(cfg, layer_specs=tuple(specs)), out

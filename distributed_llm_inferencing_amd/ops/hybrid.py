@@ -174,13 +174,14 @@ def concat_cast(a: torch.Tensor, b: torch.Tensor, dtype) -> torch.Tensor:
     return out
 
 
-_ACT_KINDS = {"gelu_mul": 0, "silu_mul": 1, "gelu": 2}
+_ACT_KINDS = {"gelu_mul": 0, "silu_mul": 1, "gelu": 2, "gelu_erf": 3, "copy": 4}
 
 
 def act_mul(gu: torch.Tensor, F_: int, dtype, kind: str = "gelu_mul",
             rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The feed-forward's middle for an fp32 projection: ``gelu_mul`` / ``silu_mul`` =
-    act(gu[:, :F]) * gu[:, F:2F]; ``gelu`` = gelu_tanh(gu[:, :F]). ``rows`` (device int32
+    act(gu[:, :F]) * gu[:, F:2F]; ``gelu`` = gelu_tanh(gu[:, :F]); ``gelu_erf`` = the exact GELU
+    of gu[:, :F]; ``copy`` = gu[:, :F] rounded to the storage dtype. ``rows`` (device int32
     scalar): only that many leading rows hold data (routed rows of a mixture)."""
     if not gu.is_cuda:
         return R.act_mul(gu, F_, dtype, kind)
@@ -378,4 +379,180 @@ def moe_finish(routed, topk_w, topk_ids, x, n_real: int, ys=None, gate=None) -> 
     _call("dli_moe_combine_f32", _p(out), None, _p(routed), _p(topk_w), None, _p(topk_ids),
           _p(x), x.stride(0), _p(ys), _p(gate), gate.stride(0) if gate is not None else 0, T,
           topk_ids.shape[1], D, n_real, _dt(x.dtype), _st())
+    return out
+
+
+# ----------------------------------------------------------------------------- post-norm designs
+def prev_tokens(ids, state, slots, cu_seqlens, max_seqlen, positions) -> torch.Tensor:
+    """int32 [T]: the token before each row (-1 at position 0). A portion's first row takes it
+    from the sequence's slot of ``state`` (int32 [slots]), which then receives the portion's
+    last token: the previous token is part of a sequence's state."""
+    if not ids.is_cuda:
+        return R.prev_tokens(ids, state, slots, cu_seqlens, positions)
+    T = ids.shape[0]
+    S = cu_seqlens.shape[0] - 1
+    prev = torch.empty(T, dtype=torch.int32, device=ids.device)
+    _call("dli_prev_tokens", _p(prev), _p(ids), _p(state), _p(slots), _p(cu_seqlens),
+          _p(positions), S, int(max_seqlen), _st())
+    return prev
+
+
+def embedding_bigram(ids, prev, table, bigram, buckets: int, mul_prev: int, mul_cur: int):
+    """(x fp32 [T, D], x rounded to the storage dtype): table[id] plus the hashed bigram row
+    (``reference.embedding_bigram``); ``bigram`` None leaves the first table alone."""
+    if not table.is_cuda:
+        return R.embedding_bigram(ids, prev, table, bigram, buckets, mul_prev, mul_cur,
+                                  table.dtype)
+    T, D = ids.shape[0], table.shape[1]
+    x = torch.empty(T, D, dtype=torch.float32, device=table.device)
+    xb = torch.empty(T, D, dtype=table.dtype, device=table.device)
+    if bigram is not None and bigram.shape[0] != buckets + 1:
+        raise ValueError("bigram table: buckets + 1 rows")
+    _call("dli_embedding_bigram", _p(x), _p(xb), _p(ids), _p(prev), _p(table), _p(bigram), T, D,
+          table.shape[0], int(buckets), int(mul_prev), int(mul_cur), _dt(table.dtype), _st())
+    return x, xb
+
+
+def postnorm(x, y, w, b, eps: float, keep: float = 1.0,
+             rows_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x = LayerNorm(keep * x + y) * w + b on the fp32 stream, in place (y optional, fp32);
+    returns the new rows in the storage dtype (w's). With ``rows_idx`` (int64) only those rows
+    are normed and returned and x is left alone."""
+    if not x.is_cuda:
+        return R.postnorm(x, y, w, b, eps, keep, w.dtype, rows_idx)
+    dim = x.shape[1]
+    rows = x.shape[0] if rows_idx is None else rows_idx.shape[0]
+    h = torch.empty(rows, dim, dtype=w.dtype, device=x.device)
+    _call("dli_postnorm", _p(x), _p(y), y.stride(0) if y is not None else 0, float(keep), _p(w),
+          _p(b), _p(h), rows, dim, float(eps), _p(rows_idx), _dt(w.dtype), _st())
+    return h
+
+
+def add_rmsnormed(x, y, w, eps: float) -> torch.Tensor:
+    """x += y / sqrt(mean(y^2) + eps) * w on the fp32 stream (y fp32); returns the new x in
+    the storage dtype."""
+    if not x.is_cuda:
+        return R.add_rmsnormed(x, y, w, eps, w.dtype)
+    rows, dim = x.shape
+    h = torch.empty(rows, dim, dtype=w.dtype, device=x.device)
+    _call("dli_add_rmsnormed", _p(x), _p(y), y.stride(0), _p(w), _p(h), rows, dim, float(eps),
+          _dt(w.dtype), _st())
+    return h
+
+
+def side_gate(gate, ids, table, col0: int) -> torch.Tensor:
+    """gelu_tanh(gate) * table[id, col0 : col0 + n] for the fp32 projection gate [T, n], in the
+    storage dtype (the table's)."""
+    if not gate.is_cuda:
+        return R.side_gate(gate, ids, table, col0, table.dtype)
+    T, n = gate.shape
+    out = torch.empty(T, n, dtype=table.dtype, device=gate.device)
+    _call("dli_side_gate", _p(out), _p(gate), gate.stride(0), _p(ids), _p(table),
+          table.stride(0), int(col0), T, n, table.shape[0], _dt(table.dtype), _st())
+    return out
+
+
+def rmsnorm_cols(src, w, eps: float) -> torch.Tensor:
+    """RMS norm times w of the rows of an fp32 matrix that may be a column slice of a wider
+    one; storage dtype out."""
+    if not src.is_cuda:
+        return R.rmsnorm_cols(src, w, eps, w.dtype)
+    T, n = src.shape
+    out = torch.empty(T, n, dtype=w.dtype, device=src.device)
+    _call("dli_rmsnorm_cols", _p(out), _p(src), src.stride(0), _p(w), T, n, float(eps),
+          _dt(w.dtype), _st())
+    return out
+
+
+def latent_prepare(qproj, kvproj, cw, eps, H, d, dr, r, rot_dims, inv_freq, positions, slots,
+                   cache, dtype, half: bool):
+    """Query / cache preparation of latent attention with the queries and the compressed kv in
+    separate fp32 projections (``reference.latent_prepare``); ``kvproj`` None: the cache is
+    another layer's and nothing is written. Returns (q_nope [T, H, d], q_full [T, H, r + dr])
+    with q_full's rotated tail written."""
+    T = qproj.shape[0]
+    if not qproj.is_cuda:
+        qn, qr = R.latent_prepare(qproj, kvproj, cw, eps, H, d, dr, r, rot_dims, inv_freq,
+                                  positions, slots, cache, dtype, half)
+        qf = torch.zeros(T, H, r + dr, dtype=dtype)
+        qf[:, :, r:] = qr
+        return qn, qf
+    qn = torch.empty(T, H, d, dtype=dtype, device=qproj.device)
+    qf = torch.empty(T, H, r + dr, dtype=dtype, device=qproj.device)
+    own = kvproj is not None
+    _call("dli_latent_prepare", _p(qproj), qproj.stride(0), _p(kvproj),
+          kvproj.stride(0) if own else 0, _p(cw) if own else None, float(eps), T, H, d, dr, r,
+          rot_dims, _p(inv_freq), _p(positions), _p(slots), _p(qn), _p(qf),
+          _p(cache) if own else None, int(half), _dt(dtype), _st())
+    return qn, qf
+
+
+def head_gate(o, g, dtype) -> torch.Tensor:
+    """o fp32 [T, H, n] times sigmoid(g[t, h]) (g an fp32 column slice [T, H]) -> storage
+    dtype [T, H*n]."""
+    if not o.is_cuda:
+        return R.head_gate(o, g, dtype)
+    T, H, n = o.shape
+    out = torch.empty(T, H * n, dtype=dtype, device=o.device)
+    _call("dli_head_gate", _p(out), _p(o), _p(g), g.stride(0), T, H, n, _dt(dtype), _st())
+    return out
+
+
+def gla(proj, z, a_bias, tau: float, norm_w, eps, state, slots, cu_seqlens, max_seqlen,
+        positions, H, d, dv):
+    """Gated linear attention over per-sequence state slots (``reference.gla``): proj fp32
+    [T, q | k | v | gate | ...], z fp32 [T, H*d]; returns the normed, gated read-out
+    [T, H*dv] in the storage dtype."""
+    dtype = norm_w.dtype
+    if not proj.is_cuda:
+        return R.gla(proj, z, a_bias, tau, norm_w, eps, state, slots, cu_seqlens, positions,
+                     H, d, dv, dtype)
+    T = proj.shape[0]
+    S = cu_seqlens.shape[0] - 1
+    out = torch.empty(T, H * dv, dtype=dtype, device=proj.device)
+    _call("dli_gla", _p(proj), proj.stride(0), _p(z), z.stride(0), _p(a_bias), float(1.0 / tau),
+          float(d ** -0.5), _p(norm_w), float(eps), _p(state), _p(slots), _p(cu_seqlens),
+          _p(positions), _p(out), out.stride(0), S, int(max_seqlen), H, d, dv, _dt(dtype), _st())
+    return out
+
+
+def logit_router(h, w_router, bias, top: int):
+    """(weights fp32 [T, top], ids int32 [T, top]): fp32 logits h . w + bias, the ``top``
+    largest chosen (lowest index on ties), softmax over the chosen ones."""
+    if not h.is_cuda:
+        return R.logit_router(h, w_router, bias, top)
+    T, D = h.shape
+    n = w_router.shape[0]
+    w = torch.empty(T, top, dtype=torch.float32, device=h.device)
+    ids = torch.empty(T, top, dtype=torch.int32, device=h.device)
+    _call("dli_logit_router", _p(w), _p(ids), _p(h), h.stride(0), _p(w_router), _p(bias), T, D,
+          n, top, _dt(h.dtype), _st())
+    return w, ids
+
+
+def moe_gelu_experts_f32(x, w_up, w_down, topk_w, topk_ids, shared=None) -> torch.Tensor:
+    """Weighted sum of every token's chosen ungated experts down(gelu_erf(up x)) in fp32, as
+    grouped GEMMs over the rows sorted by expert; ``shared`` = (ws_up, ws_down) adds the
+    always-on expert. No host synchronisation."""
+    if not x.is_cuda:
+        return R.moe_gelu_experts_f32(x, w_up, w_down, topk_w, topk_ids, shared)
+    T, D = x.shape
+    k = topk_ids.shape[1]
+    E, F_, _ = w_up.shape
+    n = T * k
+    dev = x.device
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    pos = torch.empty(n, dtype=torch.int32, device=dev)
+    src = torch.empty(max(n, 1), dtype=torch.int32, device=dev)
+    _call("dli_moe_align", _p(offsets), _p(pos), _p(src), _p(topk_ids), n, k, 0, E, _st())
+    up = grouped_linear_any(x, w_up, offsets, src, n)
+    act = act_mul(up, F_, x.dtype, "gelu_erf", rows=offsets[E:])
+    y = grouped_linear_any(act, w_down, offsets, None, n)
+    ys = None
+    if shared is not None:
+        a = act_mul(linear_any(x, shared[0]), shared[0].shape[0], x.dtype, "gelu_erf")
+        ys = linear_any(a, shared[1])
+    out = torch.empty(T, D, dtype=torch.float32, device=dev)
+    _call("dli_moe_combine_f32", _p(out), _p(y), None, _p(topk_w), _p(pos), _p(topk_ids), _p(x),
+          x.stride(0), _p(ys), None, 0, T, k, D, E, _dt(x.dtype), _st())
     return out

@@ -396,10 +396,15 @@ def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
 
 def act_mul(gu: torch.Tensor, F_: int, out_dtype: torch.dtype, kind: str) -> torch.Tensor:
     """The feed-forward's middle, fp32 in: ``gelu_mul`` / ``silu_mul`` = act(gu[:, :F]) *
-    gu[:, F:2F]; ``gelu`` = gelu_tanh(gu[:, :F])."""
+    gu[:, F:2F]; ``gelu`` = gelu_tanh(gu[:, :F]); ``gelu_erf`` = the exact GELU of gu[:, :F];
+    ``copy`` = gu[:, :F] itself."""
     g = gu[:, :F_].float()
     if kind == "gelu":
         return F.gelu(g, approximate="tanh").to(out_dtype)
+    if kind == "gelu_erf":
+        return F.gelu(g).to(out_dtype)
+    if kind == "copy":
+        return g.to(out_dtype)
     u = gu[:, F_:2 * F_].float()
     a = F.gelu(g, approximate="tanh") if kind == "gelu_mul" else F.silu(g)
     return (a * u).to(out_dtype)
@@ -616,4 +621,172 @@ def moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared=None):
         a = act_mul(linear(x, ws_gu, out_dtype=torch.float32), ws_gu.shape[0] // 2, x.dtype,
                     "silu_mul")
         out += gate.float().reshape(T, 1) * linear(a, ws_down, out_dtype=torch.float32)
+    return out
+
+
+# ----------------------------------------------------------------------------- post-norm designs
+def prev_tokens(ids, state, slots, cu_seqlens, positions):
+    """The token before each row of a step: the row above inside a portion, the sequence's slot
+    of ``state`` (int32 [slots]) for a portion's first row, -1 at position 0. The slot then
+    receives the portion's last token."""
+    prev = torch.full_like(ids, -1)
+    cu, sl = cu_seqlens.tolist(), slots.tolist()
+    for s in range(len(cu) - 1):
+        t0, t1 = cu[s], cu[s + 1]
+        if t1 <= t0 or sl[s] < 0:
+            continue
+        prev[t0 + 1:t1] = ids[t0:t1 - 1]
+        if int(positions[t0]) != 0:
+            prev[t0] = state[sl[s]]
+        state[sl[s]] = ids[t1 - 1]
+    return prev
+
+
+def embedding_bigram(ids, prev, table, bigram, buckets, mul_prev, mul_cur, out_dtype):
+    """fp32 rows table[id] + bigram[(prev * mul_prev + id * mul_cur) mod buckets] (row
+    ``buckets`` where prev < 0; ``bigram`` None: the first table alone), and their rounding to
+    ``out_dtype``."""
+    x = table[ids.long()].float()
+    if bigram is not None:
+        row = (prev.long() * mul_prev + ids.long() * mul_cur) % buckets
+        row = torch.where(prev < 0, torch.full_like(row, buckets), row)
+        x = x + bigram[row].float()
+    return x, x.to(out_dtype)
+
+
+def postnorm(x, y, w, b, eps, keep, out_dtype, rows_idx=None):
+    """Layer norm with weight and bias of keep * x + y (y optional) over the fp32 stream x, in
+    place; returns the new rows rounded to ``out_dtype``. With ``rows_idx`` only those rows are
+    normed and returned, and x stays as it is."""
+    src = x if rows_idx is None else x.index_select(0, rows_idx)
+    v = src.float() * keep
+    if y is not None:
+        v = v + y.float()
+    mu = v.mean(-1, keepdim=True)
+    var = (v - mu).pow(2).mean(-1, keepdim=True)
+    n = (v - mu) * torch.rsqrt(var + eps) * w.float() + b.float()
+    if rows_idx is None:
+        x.copy_(n)
+    return n.to(out_dtype)
+
+
+def add_rmsnormed(x, y, w, eps, out_dtype):
+    """x += y / sqrt(mean(y^2) + eps) * w on the fp32 stream, in place; returns the new x
+    rounded to ``out_dtype``."""
+    yy = y.float()
+    x.add_(yy * torch.rsqrt(yy.pow(2).mean(-1, keepdim=True) + eps) * w.float())
+    return x.to(out_dtype)
+
+
+def side_gate(gate, ids, table, col0, out_dtype):
+    """gelu_tanh(gate) * table[id, col0 : col0 + n] for an fp32 projection gate [T, n]."""
+    n = gate.shape[1]
+    e = table[ids.long()][:, col0:col0 + n].float()
+    return (F.gelu(gate.float(), approximate="tanh") * e).to(out_dtype)
+
+
+def rmsnorm_cols(src, w, eps, out_dtype):
+    """Rows of the fp32 (column-sliced) matrix ``src`` divided by their RMS, times w."""
+    v = src.float()
+    return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def rotate_pairs(x, positions, inv_freq, rot_dims, half):
+    """``half``: dimension i < rot_dims/2 pairs with i + rot_dims/2; else pairs (2i, 2i+1)."""
+    if not half:
+        return rotate_interleaved(x, positions, inv_freq, rot_dims)
+    h = rot_dims // 2
+    ang = positions.to(inv_freq.dtype)[:, None] * inv_freq[None, :]
+    c, s = ang.cos().float(), ang.sin().float()
+    if x.dim() == 3:
+        c, s = c[:, None, :], s[:, None, :]
+    out = x.clone()
+    u, v = x[..., :h], x[..., h:rot_dims]
+    out[..., :h] = u * c - v * s
+    out[..., h:rot_dims] = v * c + u * s
+    return out
+
+
+def latent_prepare(qproj, kvproj, cw, eps, H, d, dr, r, rot_dims, inv_freq, positions, slots,
+                   cache, out_dtype, half):
+    """qproj fp32 [T, H*(d+dr)] (heads laid out [d unrotated | dr rotated]); kvproj fp32
+    [T, r + dr] = [latent | shared key to rotate] or None (the layer reads another layer's
+    cache and writes nothing). Cache row = [normed latent | rotated key]. Returns
+    (q_nope [T, H, d], q_rot [T, H, dr])."""
+    T = qproj.shape[0]
+    q = qproj.float().reshape(T, H, d + dr)
+    if kvproj is not None:
+        c = kvproj[:, :r].float()
+        c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * cw.float()
+        kr = rotate_pairs(kvproj[:, r:r + dr].float(), positions, inv_freq, rot_dims, half)
+        ok = slots >= 0
+        cache[slots[ok].long()] = torch.cat([c, kr], 1)[ok].to(cache.dtype)
+    qr = rotate_pairs(q[:, :, d:], positions, inv_freq, rot_dims, half)
+    return q[:, :, :d].to(out_dtype).contiguous(), qr.to(out_dtype)
+
+
+def head_gate(o, g, out_dtype):
+    """o fp32 [T, H, n] times sigmoid(g [T, H]) per head -> [T, H*n]."""
+    T, H, n = o.shape
+    return (o.float() * torch.sigmoid(g.float())[:, :, None]).reshape(T, H * n).to(out_dtype)
+
+
+def gla(proj, z, a_bias, tau, norm_w, eps, state, slots, cu_seqlens, positions, H, d, dv,
+        out_dtype):
+    """Gated linear attention. proj fp32 [T, 2*H*d + 2*H*dv (+ ...)] = [q | k | v | gate];
+    z fp32 [T, H*d] the decay's pre-activation (its bias ``a_bias`` is added here). Per head
+    S = diag(alpha) S + k v^T with alpha = sigmoid(z + b)^(1/tau), o = S^T (q / sqrt(d)); o is
+    RMS-normed over dv times norm_w, then times silu(gate). state fp32 [slots, H, d, dv] is
+    updated in place; a portion whose first position is 0 starts from zero."""
+    T = proj.shape[0]
+    out = torch.zeros(T, H * dv, dtype=torch.float32, device=proj.device)
+    cu, sl = cu_seqlens.tolist(), slots.tolist()
+    nw = norm_w.float()
+    for s in range(len(cu) - 1):
+        t0, t1 = cu[s], cu[s + 1]
+        if t1 <= t0 or sl[s] < 0:
+            continue
+        S = state[sl[s]].clone()
+        if int(positions[t0]) == 0:
+            S.zero_()
+        p = proj[t0:t1].float()
+        qv = p[:, :H * d].reshape(-1, H, d) * (d ** -0.5)
+        kv = p[:, H * d:2 * H * d].reshape(-1, H, d)
+        vv = p[:, 2 * H * d:2 * H * d + H * dv].reshape(-1, H, dv)
+        gv = p[:, 2 * H * d + H * dv:2 * H * d + 2 * H * dv]
+        la = -F.softplus(-(z[t0:t1].float() + a_bias.float())) / tau      # log of the decay
+        av = torch.exp(la).reshape(-1, H, d)
+        for t in range(t1 - t0):
+            S = av[t][:, :, None] * S + kv[t][:, :, None] * vv[t][:, None, :]
+            o = torch.einsum("hdv,hd->hv", S, qv[t])
+            o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * nw
+            out[t0 + t] = o.reshape(H * dv) * F.silu(gv[t])
+        state[sl[s]] = S
+    return out.to(out_dtype)
+
+
+def logit_router(h, w_router, bias, top):
+    """Router logits h @ w_router^T + bias in fp32; the ``top`` largest are chosen (lowest
+    index on ties) and weighted by the softmax over the chosen logits only. Returns (weights
+    fp32 [T, top], ids int32 [T, top])."""
+    z = h.float() @ w_router.float().t() + bias.float()
+    order = torch.sort(z, dim=-1, descending=True, stable=True)
+    return torch.softmax(order.values[:, :top], -1), order.indices[:, :top].to(torch.int32)
+
+
+def moe_gelu_experts_f32(x, w_up, w_down, topk_w, topk_ids, shared=None):
+    """Weighted sum of each token's chosen ungated experts down(gelu_erf(up x)), fp32 out;
+    ``shared`` = (ws_up, ws_down) adds an always-on expert of the same form."""
+    T, D = x.shape
+    out = torch.zeros(T, D, dtype=torch.float32, device=x.device)
+    for e in range(w_up.shape[0]):
+        rows, slot = (topk_ids == e).nonzero(as_tuple=True)
+        if rows.numel() == 0:
+            continue
+        a = F.gelu(linear(x[rows], w_up[e], out_dtype=torch.float32)).to(x.dtype)
+        out.index_add_(0, rows, linear(a, w_down[e], out_dtype=torch.float32)
+                       * topk_w[rows, slot][:, None])
+    if shared is not None:
+        a = F.gelu(linear(x, shared[0], out_dtype=torch.float32)).to(x.dtype)
+        out += linear(a, shared[1], out_dtype=torch.float32)
     return out
