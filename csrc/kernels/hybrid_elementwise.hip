@@ -15,8 +15,8 @@
 //  * talk_prepare       q / k / v bias, unit-RMS q and k heads, k and v -> cache, queries with
 //                       the pre-softmax head mixing folded in -> S
 //  * concat_cast        [x ; x0] fp32 -> S rows of width 2D (the operand of the loop-entry GEMM)
-//  * act_mul            gelu_tanh(gate) * up, silu(gate) * up or gelu_tanh(up) over a fp32
-//                       projection -> S [T, F]
+//  * act_mul            gelu_tanh(gate) * up, silu(gate) * up, gelu_tanh(up), gelu_erf(up) or a
+//                       plain copy over a fp32 projection -> S [T, F]
 //  * attn_prepare       per-head RMS norm of q and k (shared weights), normed k -> key cache,
 //                       raw k -> value cache ("values are the keys"), normed q -> S
 //  * mla_prepare        latent attention: RMS norm of the compressed kv -> cache, interleaved
@@ -186,10 +186,13 @@ __device__ __forceinline__ float gelu_tanh32(float z) {
 __device__ __forceinline__ float act_pair(int kind, float g, float u) {
   if (kind == 0) return gelu_tanh32(g) * u;
   if (kind == 1) return g / (1.f + expf(-g)) * u;
+  if (kind == 3) return 0.5f * g * (1.f + erff(g * 0.7071067811865476f));
+  if (kind == 4) return g;
   return gelu_tanh32(g);
 }
 
-// kind 0: gelu_tanh(gu[:, c]) * gu[:, F + c]; 1: silu(..) * ..; 2: gelu_tanh(gu[:, c]).
+// kind 0: gelu_tanh(gu[:, c]) * gu[:, F + c]; 1: silu(..) * ..; 2: gelu_tanh(gu[:, c]);
+// 3: the exact (erf) GELU of gu[:, c]; 4: gu[:, c] itself (a rounding copy of a column slice).
 // nrows (nullable, device): rows from *nrows on hold no data and are skipped.
 template <typename S>
 __global__ void __launch_bounds__(256) act_mul_kernel(
@@ -200,7 +203,7 @@ __global__ void __launch_bounds__(256) act_mul_kernel(
   const int t = (int)(gid / F), c = (int)(gid % F);
   if (nrows != nullptr && t >= *nrows) return;
   const float* r = gu + (long)t * ldg;
-  stf(out + (long)t * ldo + c, act_pair(kind, r[c], kind == 2 ? 0.f : r[F + c]));
+  stf(out + (long)t * ldo + c, act_pair(kind, r[c], kind >= 2 ? 0.f : r[F + c]));
 }
 
 // 4 features a thread (F, ldg multiples of 4, 16-byte aligned rows): 16-byte loads
@@ -216,7 +219,7 @@ __global__ void __launch_bounds__(256) act_mul4_kernel(
   const float* r = gu + (long)t * ldg;
   const f32x4 g = *reinterpret_cast<const f32x4*>(r + c);
   f32x4 u = f32x4{0.f, 0.f, 0.f, 0.f};
-  if (kind != 2) u = *reinterpret_cast<const f32x4*>(r + F + c);
+  if (kind < 2) u = *reinterpret_cast<const f32x4*>(r + F + c);
 #pragma unroll
   for (int i = 0; i < 4; ++i) stf(out + (long)t * ldo + c + i, act_pair(kind, g[i], u[i]));
 }
@@ -325,18 +328,18 @@ __global__ void __launch_bounds__(256) attn_prepare_kernel(
 //  cache row (width r + dr): [normed latent | rotated key]
 //  q_nope [T, H, d] (S): operand of the per-head absorb GEMM
 //  q_full [T, H, r + dr] (S): this kernel writes the rotated tail [r, r+dr) of every head
-// inv_freq [rot_dims / 2] fp32; pairs (2i, 2i+1) of the first rot_dims of the dr part rotate.
+// inv_freq [rot_dims / 2] fp64; pairs (2i, 2i+1) of the first rot_dims of the dr part rotate.
 template <typename S>
 __global__ void __launch_bounds__(256) mla_prepare_kernel(
     const float* __restrict__ proj, int ldp, const S* __restrict__ cw, float eps, int T, int H,
-    int d, int dr, int r, int rot_dims, const float* __restrict__ inv_freq,
+    int d, int dr, int r, int rot_dims, const double* __restrict__ inv_freq,
     const int* __restrict__ positions, const int* __restrict__ slots, S* __restrict__ q_nope,
     S* __restrict__ q_full, S* __restrict__ cache) {
   __shared__ float red[16];
   const int t = blockIdx.x;
   const float* row = proj + (long)t * ldp;
   const float* dkv = row + (long)H * (d + dr);
-  const float pos = (float)positions[t];
+  const double pos = (double)positions[t];
   const int slot = slots[t];
   float s = 0.f;
   for (int c = threadIdx.x; c < r; c += blockDim.x) { const float v = dkv[c]; s += v * v; }
@@ -348,8 +351,8 @@ __global__ void __launch_bounds__(256) mla_prepare_kernel(
     for (int c = threadIdx.x; c < dr; c += blockDim.x) {
       float v = dkv[r + c];
       if (c < rot_dims) {
-        const float a = pos * inv_freq[c >> 1];
-        const float cs = cosf(a), sn = sinf(a);
+        const double a = pos * inv_freq[c >> 1];   // the angle in double, rounded once
+        const float cs = (float)cos(a), sn = (float)sin(a);
         const float o = dkv[r + (c ^ 1)];
         v = (c & 1) ? v * cs + o * sn : v * cs - o * sn;
       }
@@ -364,8 +367,8 @@ __global__ void __launch_bounds__(256) mla_prepare_kernel(
     } else {
       const int cc = c - d;
       if (cc < rot_dims) {
-        const float a = pos * inv_freq[cc >> 1];
-        const float cs = cosf(a), sn = sinf(a);
+        const double a = pos * inv_freq[cc >> 1];
+        const float cs = (float)cos(a), sn = (float)sin(a);
         const float o = row[h * (d + dr) + d + (cc ^ 1)];
         v = (cc & 1) ? v * cs + o * sn : v * cs - o * sn;
       }
@@ -451,7 +454,7 @@ extern "C" int dli_token_shift(const float* h, const void* mu, float* state, con
 extern "C" int dli_act_mul(void* out, int ldo, const float* gu, int ldg, int T, int F, int kind,
                            const int* nrows, int dt, hipStream_t st) {
   if (T <= 0) return 0;
-  if (kind < 0 || kind > 2) return (int)hipErrorInvalidValue;
+  if (kind < 0 || kind > 4) return (int)hipErrorInvalidValue;
   if (F % 4 == 0 && ldg % 4 == 0 && (uintptr_t)gu % 16 == 0) {
     const int nb4 = (int)(((long)T * (F / 4) + 255) / 256);
     DT_SWITCH(dt,
@@ -506,7 +509,7 @@ extern "C" int dli_attn_prepare(const float* proj, int ldp, const void* qw, cons
 }
 
 extern "C" int dli_mla_prepare(const float* proj, int ldp, const void* cw, float eps, int T,
-                               int H, int d, int dr, int r, int rot_dims, const float* inv_freq,
+                               int H, int d, int dr, int r, int rot_dims, const double* inv_freq,
                                const int* positions, const int* slots, void* q_nope,
                                void* q_full, void* cache, int dt, hipStream_t st) {
   if (T <= 0) return 0;

@@ -503,6 +503,7 @@ __global__ void __launch_bounds__(256) score_router_kernel(
 }
 
 // out[t] = sum_j w[t][j] * (routed ? y[pos[t][j]] : identity ? x[t] : 0) + gate[t] * ys[t]
+// (gate null: the shared part is added as it is)
 // y, ys fp32; x storage type; ids >= n_real are identity experts (their pos is -1). With
 // `routed` (storage type [T, dim]: the real experts' weighted sum, already combined) instead
 // of y / pos, only the identity and shared parts are added to it.
@@ -523,7 +524,7 @@ __global__ void __launch_bounds__(256) moe_combine_f32_kernel(
     if (p >= 0) acc += ww * y[(long)p * dim + c];
     else if (ids[t * k + j] >= n_real) acc += ww * rld(x + (long)t * ldx + c);
   }
-  if (ys != nullptr) acc += gate[(long)t * ldg] * ys[(long)t * dim + c];
+  if (ys != nullptr) acc += (gate != nullptr ? gate[(long)t * ldg] : 1.f) * ys[(long)t * dim + c];
   out[gid] = acc;
 }
 
@@ -553,7 +554,7 @@ extern "C" int dli_moe_combine_f32(float* out, const float* y, const void* route
                                    int ldx, const float* ys, const float* gate, int ldg, int T,
                                    int k, int dim, int n_real, int dt, hipStream_t st) {
   if (T <= 0) return 0;
-  if ((ys == nullptr) != (gate == nullptr) || (y == nullptr) != (pos == nullptr) ||
+  if ((ys == nullptr && gate != nullptr) || (y == nullptr) != (pos == nullptr) ||
       (y == nullptr) == (routed == nullptr))
     return (int)hipErrorInvalidValue;
   const int nb = (int)(((long)T * dim + 255) / 256);

@@ -90,6 +90,17 @@ _SIGS = {
                                   I, I, I, I, I, I, I, I, I, F, I, P, I, I, I, P],
     "dli_window_attention_mfma_workspace_bytes": [I, I, I, I, I, I, I, I],
     "dli_hgrn2": [P, I, P, P, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P],
+    "dli_gla": [P, I, P, I, P, F, F, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P],
+    # post-norm designs (postnorm.hip)
+    "dli_prev_tokens": [P, P, P, P, P, P, I, I, P],
+    "dli_embedding_bigram": [P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+    "dli_postnorm": [P, P, I, F, P, P, P, I, I, F, P, I, P],
+    "dli_add_rmsnormed": [P, P, I, P, P, I, I, F, I, P],
+    "dli_side_gate": [P, P, I, P, P, I, I, I, I, I, I, P],
+    "dli_rmsnorm_cols": [P, P, I, P, I, I, F, I, P],
+    "dli_latent_prepare": [P, I, P, I, P, F, I, I, I, I, I, I, P, P, P, P, P, P, I, I, P],
+    "dli_head_gate": [P, P, P, I, I, I, I, I, P],
+    "dli_logit_router": [P, P, P, I, P, P, I, I, I, I, I, P],
 }
 
 
