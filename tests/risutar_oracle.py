@@ -192,3 +192,116 @@ def forward(cfg, sd, tokens, trace=None):
             trace.append(x.clone())
     x = layer_norm(x, sd["final.norm"], sd["final.norm.b"], eps)
     return x @ f64(sd["head"]).T
+
+
+# ----------------------------------------------------------------------------- test models
+def tensor_shapes(cfg, decay_rank=6):
+    """Checkpoint tensor names and shapes of a configuration."""
+    D, V = cfg["width"], cfg["vocab"]
+    out = {"embed": (V, D), "final.norm": (D,), "final.norm.b": (D,), "head": (V, D)}
+    bg = (cfg.get("embedding") or {}).get("bigram")
+    if bg:
+        out["bigram"] = (bg["buckets"] + 1, D)
+    side = (cfg.get("token_side") or {}).get("dim", 0)
+    if side:
+        out["side.embed"] = (V, side * len(cfg["layers"]))
+    for i, L in enumerate(cfg["layers"]):
+        a, m = f"l{i}.", L["mixer"]
+        for n in ("norm1", "norm2") if L.get("mlp") else ("norm1",):
+            out[a + n] = (D,)
+            out[a + n + ".b"] = (D,)
+        H = m["heads"]
+        if L["type"] == "gla":
+            d, dv = m["dim"], m["vdim"]
+            out.update({a + "mix.q": (H * d, D), a + "mix.k": (H * d, D), a + "mix.v": (H * dv, D),
+                        a + "mix.g": (H * dv, D), a + "mix.o": (D, H * dv), a + "mix.norm": (dv,),
+                        a + "mix.a1": (decay_rank, D), a + "mix.a2": (H * d, decay_rank),
+                        a + "mix.a2.b": (H * d,)})
+        else:
+            d, dr, dv, r, rq = m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            out.update({a + "mix.dq": (rq, D), a + "mix.dq.norm": (rq,),
+                        a + "mix.uq": (H * (d + dr), rq), a + "mix.uk": (H * d, r),
+                        a + "mix.uv": (H * dv, r), a + "mix.g": (H, D), a + "mix.o": (D, H * dv)})
+            if m.get("kv_from") is None:
+                out.update({a + "mix.dkv": (r + dr, D), a + "mix.dkv.norm": (r,)})
+        mlp = L.get("mlp")
+        if mlp and mlp["kind"] == "dense":
+            F = mlp["ff"]
+            out.update({a + "mlp.gate": (F, D), a + "mlp.up": (F, D), a + "mlp.down": (D, F)})
+        elif mlp:
+            F = mlp["expert"]["ff"]
+            E = mlp["router"]["experts"]
+            out.update({a + "mlp.router": (E, D), a + "mlp.router.b": (E,)})
+            for e in range(E):
+                out.update({f"{a}mlp.e{e}.up": (F, D), f"{a}mlp.e{e}.down": (D, F)})
+            if mlp.get("shared"):
+                Fs = mlp["shared"]["ff"]
+                out.update({a + "mlp.shared.up": (Fs, D), a + "mlp.shared.down": (D, Fs)})
+        if side:
+            out.update({a + "side.gate": (side, D), a + "side.proj": (D, side),
+                        a + "side.norm": (D,)})
+    return out
+
+
+def bf16_exact(t):
+    """Round to values bfloat16 holds exactly (so that a bf16 and an fp32 copy agree)."""
+    return t.to(torch.float32).to(torch.bfloat16).to(F64)
+
+
+def random_weights(cfg, seed=0, decay_rank=6):
+    """Random float64 weights that bfloat16 holds exactly, sized so that every mechanism
+    matters: norm weights and biases away from 1 and 0, router biases, decays spread between
+    fast and slow, side inputs and bigram rows as large as the embedding."""
+    g = torch.Generator().manual_seed(seed)
+    w = {}
+    for name, shape in tensor_shapes(cfg, decay_rank).items():
+        rn = torch.randn(shape, generator=g, dtype=F64)
+        if name.endswith((".norm1", ".norm2", "final.norm", ".dq.norm", ".dkv.norm", "mix.norm",
+                          "side.norm")):
+            v = 0.7 + 0.6 * torch.rand(shape, generator=g, dtype=F64)
+        elif name.endswith("a2.b"):
+            v = 1.5 + 2.0 * rn
+        elif name.endswith(".b"):
+            v = 0.3 * rn
+        elif name in ("embed", "bigram", "side.embed"):
+            v = rn
+        elif name.endswith("mlp.router"):
+            v = 2.0 * rn / math.sqrt(shape[-1])
+        elif name.endswith("mix.a2"):
+            v = 2.0 * rn / math.sqrt(shape[-1])
+        else:
+            v = rn / math.sqrt(shape[-1])
+        w[name] = bf16_exact(v)
+    return w
+
+
+def route_margins(cfg, sd, tokens):
+    """Per position, the smallest gap between the last chosen and the first rejected router
+    logit over all routed layers (a small gap: a close call that rounding may turn)."""
+    eps, alpha = cfg["norm"]["eps"], cfg["postln_alpha"]
+    T = len(tokens)
+    gaps = torch.full((T,), float("inf"), dtype=F64)
+    trace = []
+    forward(cfg, sd, tokens, trace)
+    # replay the layers to reach each feed-forward's input
+    x = embed(cfg, sd, tokens)
+    kvs = {}
+    for i, L in enumerate(cfg["layers"]):
+        pre, m = f"l{i}.", L["mixer"]
+        if L["type"] == "latent_attention":
+            src = m.get("kv_from")
+            if src is None:
+                kvs[i] = latent_kv(m, sd, pre + "mix.", x, eps)
+                src = i
+            y = latent_attention(m, sd, pre + "mix.", x, eps, kvs[src])
+        else:
+            y = gla(m, sd, pre + "mix.", x, eps)
+        x = layer_norm(alpha * x + y, sd[pre + "norm1"], sd[pre + "norm1.b"], eps)
+        mlp = L.get("mlp")
+        if mlp and mlp["kind"] == "moe" and mlp["router"]["top"] < mlp["router"]["experts"]:
+            z = x @ f64(sd[pre + "mlp.router"]).T + f64(sd[pre + "mlp.router.b"])
+            s = torch.sort(z, dim=-1, descending=True).values
+            top = mlp["router"]["top"]
+            gaps = torch.minimum(gaps, s[:, top - 1] - s[:, top])
+        x = trace[i]
+    return gaps.numpy()
