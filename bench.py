@@ -67,30 +67,14 @@ def _like_for_like_value():
         return None
 
 
-def run_design_pulunex(a):
-    """``--design pulunex``: prefill and decode throughput of the design at layer sizes of a
-    real model (random weights) beside the framework's closest model, a Mixtral of equal width,
-    depth, heads, experts, expert width and experts per token, both through ``LLMEngine``."""
-    from dataclasses import replace
+def _design_sweep(cfgs, a, V):
+    """Prefill and decode throughput of every configuration in ``cfgs`` (those named in
+    ``--design-models``) through ``LLMEngine``: {config name: {measurement: value}}."""
     from distributed_llm_inferencing_amd.engine import SamplingParams
     from distributed_llm_inferencing_amd.engine.llm_engine import LLMEngine
-    from distributed_llm_inferencing_amd.models.configs import LayerSpec, get_config, hybrid_config
-    D, Fw, V, Hh, G, hd = a.design_width, a.design_ff, 32000, a.design_width // 128, 8, 128
-    E, top, chunk = 8, 2, a.design_window
-
-    def lay(kv_from=-1):
-        return LayerSpec("talk_attention", heads=Hh, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5,
-                         chunk=chunk, kv_from=kv_from, shift=True, ff_kind="moe", ff=Fw,
-                         experts=E, identity=2, top=top, shared_ff=2048)
-    hyb = hybrid_config("pulunex-bench", D, V, (lay(), lay(), lay(1), lay(1)), arch="pulunex",
-                        max_position=1 << 15, embed_scale=8.0, logit_scale=0.5, learned_pos=True,
-                        scalar_norm=True)
-    mix = replace(get_config("mixtral-8x7b"), name="mixtral-bench", hidden_size=D, num_layers=4,
-                  num_heads=Hh, num_kv_heads=G, head_dim=hd, intermediate_size=Fw, vocab_size=V,
-                  num_experts=E, top_k_experts=top, max_position=1 << 15)
     rng = np.random.default_rng(0)
     out = {}
-    for cfg in (hyb, mix):
+    for cfg in cfgs:
         if cfg.name.split("-")[0] not in a.design_models.split(","):
             continue
         res = {}
@@ -147,12 +131,74 @@ def run_design_pulunex(a):
             del eng
             torch.cuda.empty_cache()
         out[cfg.name] = res
+    return out
+
+
+def run_design_pulunex(a):
+    """``--design pulunex``: prefill and decode throughput of the design at layer sizes of a
+    real model (random weights) beside the framework's closest model, a Mixtral of equal width,
+    depth, heads, experts, expert width and experts per token, both through ``LLMEngine``."""
+    from dataclasses import replace
+    from distributed_llm_inferencing_amd.engine import SamplingParams
+    from distributed_llm_inferencing_amd.engine.llm_engine import LLMEngine
+    from distributed_llm_inferencing_amd.models.configs import LayerSpec, get_config, hybrid_config
+    D, Fw, V, Hh, G, hd = a.design_width, a.design_ff, 32000, a.design_width // 128, 8, 128
+    E, top, chunk = 8, 2, a.design_window
+
+    def lay(kv_from=-1):
+        return LayerSpec("talk_attention", heads=Hh, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5,
+                         chunk=chunk, kv_from=kv_from, shift=True, ff_kind="moe", ff=Fw,
+                         experts=E, identity=2, top=top, shared_ff=2048)
+    hyb = hybrid_config("pulunex-bench", D, V, (lay(), lay(), lay(1), lay(1)), arch="pulunex",
+                        max_position=1 << 15, embed_scale=8.0, logit_scale=0.5, learned_pos=True,
+                        scalar_norm=True)
+    mix = replace(get_config("mixtral-8x7b"), name="mixtral-bench", hidden_size=D, num_layers=4,
+                  num_heads=Hh, num_kv_heads=G, head_dim=hd, intermediate_size=Fw, vocab_size=V,
+                  num_experts=E, top_k_experts=top, max_position=1 << 15)
+    out = _design_sweep((hyb, mix), a, V)
     print(json.dumps({"metric": "prefill and decode tokens/s, Pulunex design vs Mixtral of equal "
                                 "size (random weights)", "unit": "tokens/s", "n_gpus": 1,
                       "dtype": "bf16", "data": "synthetic prompts, random-init weights",
                       "config": {"width": D, "expert_ff": Fw, "layers": 4, "heads": Hh,
                                  "kv_heads": G, "head_dim": hd, "block": chunk, "experts": E,
                                  "identity_experts": 2, "top": top, "shared_ff": 2048},
+                      "results": out}), flush=True)
+
+
+def run_design_risutar(a):
+    """``--design risutar``: prefill and decode throughput of the design at layer sizes of a
+    real model (random weights) beside the framework's closest model, a Mixtral of equal width,
+    depth, heads, expert count, experts per token and expert FLOPs (the design's experts are
+    ungated, so their width is 3/2 of the gated ones'), both through ``LLMEngine``."""
+    from dataclasses import replace
+    from distributed_llm_inferencing_amd.models.configs import LayerSpec, get_config, hybrid_config
+    D, Fw, V, Hh, G, hd = a.design_width, a.design_ff, 32000, a.design_width // 128, 8, 128
+    E, top = 8, 2
+    moe = dict(ff_kind="moe", router="logit_topk", expert_act="gelu_erf", ff=Fw * 3 // 2,
+               experts=E, top=top, shared_ff=3072)
+
+    def gla():
+        return LayerSpec("gla", heads=Hh, dim=hd, vdim=hd, tau=16.0, decay_rank=16, **moe)
+
+    def latent(kv_from=-1):
+        return LayerSpec("latent_attention", heads=Hh, kv_heads=1, dim=hd, vdim=hd,
+                         window=1 << 30, scale=(hd + 64) ** -0.5, rot_dim=64, kv_rank=512,
+                         rot_dims=64, q_rank=1536, head_gate=True, rot_half=True,
+                         kv_from=kv_from, **moe)
+    hyb = hybrid_config("risutar-bench", D, V, (gla(), latent(), latent(1), gla()),
+                        arch="risutar", max_position=1 << 15, norm_eps=1e-5, postln_alpha=3.0,
+                        bigram=(65521, 127, 7), side_dim=16)
+    mix = replace(get_config("mixtral-8x7b"), name="mixtral-bench", hidden_size=D, num_layers=4,
+                  num_heads=Hh, num_kv_heads=G, head_dim=hd, intermediate_size=Fw, vocab_size=V,
+                  num_experts=E, top_k_experts=top, max_position=1 << 15)
+    out = _design_sweep((hyb, mix), a, V)
+    print(json.dumps({"metric": "prefill and decode tokens/s, Risutar design vs Mixtral of equal "
+                                "size (random weights)", "unit": "tokens/s", "n_gpus": 1,
+                      "dtype": "bf16", "data": "synthetic prompts, random-init weights",
+                      "config": {"width": D, "expert_ff": Fw * 3 // 2, "layers": 4, "heads": Hh,
+                                 "head_dim": hd, "kv_rank": 512, "q_rank": 1536, "rot_dim": 64,
+                                 "experts": E, "top": top, "shared_ff": 3072, "side_dim": 16,
+                                 "bigram_buckets": 65521},
                       "results": out}), flush=True)
 
 
@@ -380,11 +426,11 @@ def main():
                     help="N>1: pp = layer-sharded pipeline (dense, default), ep = expert "
                          "parallel (MoE), tp = tensor-parallel ablation, dp = independent "
                          "replicas")
-    ap.add_argument("--design", default=None, choices=["buborax", "pulunex"],
+    ap.add_argument("--design", default=None, choices=["buborax", "pulunex", "risutar"],
                     help="instead of the headline workload: prefill / decode throughput of "
                          "this design at real layer sizes beside the closest model of equal "
-                         "size (buborax: Llama, pulunex: Mixtral)")
-    ap.add_argument("--design-models", default="buborax,llama,pulunex,mixtral",
+                         "size (buborax: Llama, pulunex and risutar: Mixtral)")
+    ap.add_argument("--design-models", default="buborax,llama,pulunex,mixtral,risutar",
                     help="which of the design and its comparison model to run")
     ap.add_argument("--design-width", type=int, default=4096)
     ap.add_argument("--design-ff", type=int, default=14336)
@@ -396,6 +442,8 @@ def main():
     a = ap.parse_args()
     if a.design:
         _heartbeat()
+        if a.design == "risutar":
+            return run_design_risutar(a)
         return run_design_pulunex(a) if a.design == "pulunex" else run_design(a)
 
     from distributed_llm_inferencing_amd import launch

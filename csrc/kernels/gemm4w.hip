@@ -15,5 +15,5 @@ static int dispatch_4w(int tile_cfg, DLI_GEMM_ARGS) {
   }
 }
 
-int gemm_4w_dispatch(int epi, int tile_cfg, DLI_GEMM_ARGS) { DLI_EPI_SWITCH(dispatch_4w) }
+int gemm_4w_dispatch(int epi, int tile_cfg, DLI_GEMM_ARGS) { DLI_EPI_SWITCH_BASE(dispatch_4w) }
 int gemm_4w_set_slab_store(int mode) { return set_slab_store_tu(mode); }

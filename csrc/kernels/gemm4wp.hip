@@ -277,4 +277,4 @@ static int dispatch_4wp(int tile_cfg, DLI_GEMM_ARGS) {
   return launch_4wp<EPI>(A, lda, W, ldw, C, ldc, M, N, K, splits, bias, go, st);
 }
 
-int gemm_4wp_dispatch(int epi, int tile_cfg, DLI_GEMM_ARGS) { DLI_EPI_SWITCH(dispatch_4wp) }
+int gemm_4wp_dispatch(int epi, int tile_cfg, DLI_GEMM_ARGS) { DLI_EPI_SWITCH_BASE(dispatch_4wp) }

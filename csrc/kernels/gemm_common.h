@@ -15,7 +15,9 @@ enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_SILU = 2, EPI_BIAS_GELU = 3, EPI_BIAS = 4,
        // slab-only split-K call (C == nullptr, splits > 1) whose partials are stored as fp16
        // scaled by 1/16 instead of fp32 (half the bytes the GEMM writes and its consumer
        // reads; the scale keeps |partial| up to ~1e6 in range). Tiles and 8-phase families.
-       EPI_SLAB16 = 5 };
+       EPI_SLAB16 = 5,
+       // the exact (erf) GELU of the product, no bias (ungated expert feed-forwards)
+       EPI_GELU_ERF = 6 };
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
@@ -30,6 +32,18 @@ __device__ __forceinline__ float gelu_f(float x) {
   return x / (1.f + __expf(-y2));
 }
 
+// exact GELU x * Phi(x), branch-free (see gelu_f on why): Phi(-|x|) = erfc(|x| / sqrt 2) / 2
+// by the rational-times-Gaussian form of Abramowitz & Stegun 7.1.26 (|error| < 1.5e-7
+// absolute, and relative on the negative side, where Phi itself is small), mirrored by a select
+__device__ __forceinline__ float gelu_erf_f(float x) {
+  const float z = fabsf(x) * 0.7071067811865476f;
+  const float t = 1.f / (1.f + 0.3275911f * z);
+  const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f +
+                     t * (-1.453152027f + t * 1.061405429f))));
+  const float e = 0.5f * poly * __expf(-z * z);
+  return x * (x < 0.f ? e : 1.f - e);
+}
+
 template <int EPI>
 __device__ __forceinline__ void store_pair_or_one(void* C, int ldc, int row, int col, float v,
                                                   const u16* bias) {
@@ -38,6 +52,7 @@ __device__ __forceinline__ void store_pair_or_one(void* C, int ldc, int row, int
   } else {
     if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) v += bf2f(bias[col]);
     if (EPI == EPI_BIAS_GELU) v = gelu_f(v);
+    if (EPI == EPI_GELU_ERF) v = gelu_erf_f(v);
     ((u16*)C)[(long)row * ldc + col] = f2bf(v);
   }
 }
@@ -163,6 +178,10 @@ __device__ __forceinline__ void store_quad(void* C, int ldc, int row, int col, i
 #pragma unroll
     for (int r = 0; r < 4; ++r) o[r] = gelu_f(o[r]);
   }
+  if (EPI == EPI_GELU_ERF) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[r] = gelu_erf_f(o[r]);
+  }
   uint2 pk;
   pk.x = pack2bf(o[0], o[1]);
   pk.y = pack2bf(o[2], o[3]);
@@ -284,6 +303,12 @@ int gemm_4w_set_slab_store(int mode);
   DLI_EPI_SWITCH(FN)
 
 #define DLI_EPI_SWITCH(FN)                                                         \
+  if (epi == EPI_GELU_ERF) return FN<EPI_GELU_ERF>(tile_cfg, DLI_GEMM_PASS);       \
+  DLI_EPI_SWITCH_BASE(FN)
+
+// without the exact-GELU epilogue: the 4-wave families, whose 256-accumulator epilogue does
+// not unroll with it (the accumulators would leave the AGPR file inside the K loop)
+#define DLI_EPI_SWITCH_BASE(FN)                                                    \
   switch (epi) {                                                                   \
     case EPI_BF16: return FN<EPI_BF16>(tile_cfg, DLI_GEMM_PASS);                   \
     case EPI_F32: return FN<EPI_F32>(tile_cfg, DLI_GEMM_PASS);                     \

@@ -431,6 +431,7 @@ int gemm_gemv_dispatch(int epi, int tile_cfg, DLI_GEMM_ARGS) {
     case EPI_SILU: return dispatch_gemv<EPI_SILU>(tile_cfg, A, lda, W, ldw, C, ldc, M, N, K, splits, bias, ws, st);
     case EPI_BIAS_GELU: return dispatch_gemv<EPI_BIAS_GELU>(tile_cfg, A, lda, W, ldw, C, ldc, M, N, K, splits, bias, ws, st);
     case EPI_BIAS: return dispatch_gemv<EPI_BIAS>(tile_cfg, A, lda, W, ldw, C, ldc, M, N, K, splits, bias, ws, st);
+    case EPI_GELU_ERF: return dispatch_gemv<EPI_GELU_ERF>(tile_cfg, A, lda, W, ldw, C, ldc, M, N, K, splits, bias, ws, st);
     default: return (int)hipErrorInvalidValue;
   }
 }

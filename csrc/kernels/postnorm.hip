@@ -231,7 +231,7 @@ constexpr int ROUTER_MAX = 1024;
 template <typename S>
 __global__ void __launch_bounds__(256) logit_router_kernel(
     float* __restrict__ topk_w, int* __restrict__ topk_ids, const S* __restrict__ h, int ldh,
-    const S* __restrict__ W, const float* __restrict__ bias, int D, int n, int top) {
+    const S* __restrict__ W, const float* __restrict__ bias, int D, int n, int top, bool vec) {
   extern __shared__ __attribute__((aligned(16))) float rsm[];   // [D] row, [n] logits
   float* row = rsm;
   float* z = rsm + D;
@@ -239,10 +239,36 @@ __global__ void __launch_bounds__(256) logit_router_kernel(
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
   for (int c = threadIdx.x; c < D; c += blockDim.x) row[c] = ldf(h + (long)t * ldh + c);
   __syncthreads();
+  constexpr int CH = 16 / sizeof(S);            // elements of a 16-byte load
+  const int nch = D / CH;
   for (int e = wid; e < n; e += nw) {
     const S* wr = W + (long)e * D;
     float acc = 0.f;
-    for (int c = lane; c < D; c += 64) acc += row[c] * ldf(wr + c);
+    if (vec) {                                  // 16-byte loads of the router row, 4 in flight
+      for (int c0 = lane; c0 < nch; c0 += 256) {
+        uint4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          v[u] = c0 + u * 64 < nch ? *reinterpret_cast<const uint4*>(wr + (long)(c0 + u * 64) * CH)
+                                   : uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (c0 + u * 64 >= nch) continue;
+          const float* rr = row + (c0 + u * 64) * CH;
+          if constexpr (sizeof(S) == 2) {
+            float f[8];
+            unpack8bf(v[u], f);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) acc += rr[q] * f[q];
+          } else {
+            acc += rr[0] * __uint_as_float(v[u].x) + rr[1] * __uint_as_float(v[u].y) +
+                   rr[2] * __uint_as_float(v[u].z) + rr[3] * __uint_as_float(v[u].w);
+          }
+        }
+      }
+    } else {
+      for (int c = lane; c < D; c += 64) acc += row[c] * ldf(wr + c);
+    }
     acc = wave_sum(acc);
     if (lane == 0) z[e] = acc + (bias != nullptr ? bias[e] : 0.f);
   }
@@ -399,11 +425,12 @@ extern "C" int dli_logit_router(float* topk_w, int* topk_ids, const void* h, int
   if (n < 1 || top < 1 || top > n || n > ROUTER_MAX || (size_t)(D + n) * 4 > 60000)
     return (int)hipErrorInvalidValue;
   const size_t sh = (size_t)(D + n) * 4;
+  const bool vec = (uintptr_t)W % 16 == 0 && D % (dt == 0 ? 8 : 4) == 0;
   DT_SWITCH(dt,
             (logit_router_kernel<u16><<<T, 256, sh, st>>>(topk_w, topk_ids, (const u16*)h, ldh,
-                                                          (const u16*)W, bias, D, n, top)),
+                                                          (const u16*)W, bias, D, n, top, vec)),
             (logit_router_kernel<float><<<T, 256, sh, st>>>(topk_w, topk_ids, (const float*)h,
                                                             ldh, (const float*)W, bias, D, n,
-                                                            top)));
+                                                            top, vec)));
   DLI_RETURN_LAUNCH();
 }

@@ -218,6 +218,10 @@ class HybridLM(TransformerLM):
             if "ff_tuned" in lp:
                 if spec.ff_kind == "gelu":
                     fused[id(lp["w_up"])] = "bias_gelu"
+                elif spec.ff_kind == "gated_silu":
+                    fused[id(lp["w_gu"])] = "silu_mul"
+                elif spec.shared_ff and spec.expert_act == "gelu_erf":
+                    fused[id(lp["ws_up"])] = "gelu_erf"
                 elif spec.shared_ff:
                     fused[id(lp["ws_gu"])] = "silu_mul"
         for w in mats:
@@ -235,9 +239,11 @@ class HybridLM(TransformerLM):
         out, seen = [], set()
         for spec, lp in zip(self.cfg.layer_specs, self.layers):
             if spec.ff_kind == "moe" and "ff_tuned" in lp:
-                key = (tuple(lp["w_gu"].shape), spec.top)
+                w1, epi = ((lp["w_up"], "gelu_erf") if spec.expert_act == "gelu_erf"
+                           else (lp["w_gu"], "silu_mul"))
+                key = (tuple(w1.shape), spec.top, epi)
                 if key not in seen:
                     seen.add(key)
                     rows = M * spec.top
-                    out += [(rows, lp["w_gu"], "silu_mul"), (rows, lp["w_down"], "none")]
+                    out += [(rows, w1, epi), (rows, lp["w_down"], "none")]
         return out

@@ -167,17 +167,21 @@ MIXERS = {"attention": attention_mixer, "hgrn2": hgrn2_mixer,
 # framework's other mixture model.
 def prepare_feed_forward(spec: LayerSpec, params: dict, pre: str) -> None:
     """Re-lay the feed-forward weights of layer ``pre`` for the tuned GEMMs when they fit
-    (in ``params``, in place; marked by ``<pre>ff_tuned`` so that it happens once)."""
+    (in ``params``, in place; marked by ``<pre>ff_tuned`` so that it happens once). Ungated
+    experts (``expert_act`` = ``gelu_erf``) need no re-layout: their activation is an epilogue
+    of the plain weight."""
     from ..ops.reference import interleave_gate_up
     w = params.get(pre + "w_down")
     if (not spec.ff or w is None or pre + "ff_tuned" in params or w.dtype != torch.bfloat16
-            or not w.is_cuda or spec.ff_kind not in ("gelu", "moe") or spec.router != "score"
-            or w.shape[-2] % 64
-            or spec.ff % 64 or spec.shared_ff % 64):
+            or not w.is_cuda or spec.ff_kind not in ("gelu", "moe", "gated_silu")
+            or w.shape[-2] % 64 or spec.ff % 64 or spec.shared_ff % 64):
         return
     if spec.ff_kind == "gelu":
         params[pre + "b_up"] = torch.zeros(spec.ff, dtype=w.dtype, device=w.device)
-    else:
+    elif spec.ff_kind == "gated_silu":
+        gu = params[pre + "w_gu"]
+        params[pre + "w_gu"] = interleave_gate_up(gu[:spec.ff], gu[spec.ff:]).contiguous()
+    elif spec.expert_act == "silu_mul":
         gu = params[pre + "w_gu"]
         for e in range(gu.shape[0]):                 # expert by expert: no second full copy
             gu[e] = interleave_gate_up(gu[e, :spec.ff].clone(), gu[e, spec.ff:].clone())
@@ -202,7 +206,11 @@ def gelu_ff(spec: LayerSpec, lp: dict, h):
 
 
 def gated_silu_ff(spec: LayerSpec, lp: dict, h):
-    act = H.act_mul(H.linear_any(h, lp["w_gu"]), spec.ff, h.dtype, "silu_mul")
+    if "ff_tuned" in lp:
+        from .. import ops
+        act = ops.linear(h, lp["w_gu"], epi="silu_mul")
+    else:
+        act = H.act_mul(H.linear_any(h, lp["w_gu"]), spec.ff, h.dtype, "silu_mul")
     return H.linear_any(act, lp["w_down"])
 
 
@@ -212,8 +220,15 @@ def moe_ff(spec: LayerSpec, lp: dict, h):
     experts and an always-on shared expert."""
     if spec.router == "logit_topk":
         tw, ti = H.logit_router(h, lp["router"], lp["router_b"], spec.top)
-        shared = (lp["ws_up"], lp["ws_down"]) if spec.shared_ff else None
-        return H.moe_gelu_experts_f32(h, lp["w_up"], lp["w_down"], tw, ti, shared)
+        if "ff_tuned" not in lp:
+            shared = (lp["ws_up"], lp["ws_down"]) if spec.shared_ff else None
+            return H.moe_gelu_experts_f32(h, lp["w_up"], lp["w_down"], tw, ti, shared)
+        from .. import ops
+        routed = ops.moe_mlp(h, lp["w_up"], lp["w_down"], tw, ti, 0, act="gelu_erf")
+        ys = None
+        if spec.shared_ff:
+            ys = H.linear_any(ops.linear(h, lp["ws_up"], epi="gelu_erf"), lp["ws_down"])
+        return H.moe_finish(routed, tw, ti, h, lp["w_up"].shape[0], ys, None)
     ng = 1 if spec.shared_ff else 0
     tw, ti, gates = H.score_router(h, lp["router"], lp["correction"], spec.top, ng)
     if "ff_tuned" not in lp:

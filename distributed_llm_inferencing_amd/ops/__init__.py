@@ -237,7 +237,7 @@ def _gemm_native(x, w, epi: str, bias=None, out=None, plan: Optional[G.GemmPlan]
 
 
 def linear(x, w, bias=None, epi: str = "none", out=None):
-    """y = epi(x @ w.T (+bias)). epi in {none, f32, silu_mul, bias_gelu, bias}.
+    """y = epi(x @ w.T (+bias)). epi in {none, f32, silu_mul, bias_gelu, bias, gelu_erf}.
     silu_mul expects the 16-row interleaved gate/up weight and returns width N/2."""
     if bias is not None and epi == "none":
         epi = "bias"
@@ -257,6 +257,8 @@ def linear(x, w, bias=None, epi: str = "none", out=None):
             y = R.linear(x, w, out_dtype=torch.float32)
         elif epi == "bias_gelu":
             y = R.gelu_tanh(R.linear(x, w, bias))
+        elif epi == "gelu_erf":
+            y = torch.nn.functional.gelu(R.linear(x, w, out_dtype=torch.float32)).to(x.dtype)
         else:
             y = R.linear(x, w, bias)
         if out is not None:
@@ -689,19 +691,26 @@ def moe_router(h, w_router, k: int):
 
 
 def moe_mlp(x, w_gu, w_down, topk_w, topk_ids, expert_offset: int = 0,
-            plan_rows: Optional[int] = None, defer_combine: bool = False):
+            plan_rows: Optional[int] = None, defer_combine: bool = False,
+            act: str = "silu_mul"):
     """Experts [expert_offset, expert_offset+E_local) of one MoE layer; returns the weighted
     sum over the token's selected local experts (zeros for tokens routed elsewhere).
+    ``act``: ``silu_mul`` (gated experts, ``w_gu`` = the interleaved gate/up weight) or
+    ``gelu_erf`` (ungated experts down(gelu(up x)), ``w_gu`` = the up weight [E, F, D]).
     ``plan_rows``: the routed rows these experts typically receive, when ``x`` is a region
     sized for the worst case (the expert-parallel receive region: every peer's bucket at
     min(k, E/N) rows per token). The grouped-GEMM plan is looked up for it — the autotuned
     key — instead of for the capacity, whose 4-8x larger row count mapped to 256-row tiles
     (1 workgroup per CU) that streamed the experts at ~2 TB/s."""
     if not _use_native(x):
+        if act != "silu_mul":
+            raise ValueError("moe_mlp: ungated experts run on the GPU path only")
         return R.moe_mlp(x, w_gu, w_down, topk_w, topk_ids, expert_offset)
     T, D = x.shape
     k = topk_ids.shape[1]
     E_local, F2, _ = w_gu.shape
+    gated = act == "silu_mul"
+    Fa = F2 // 2 if gated else F2              # width of the activation
     n = T * k
     dev = x.device
     offsets = torch.empty(E_local + 1, dtype=torch.int32, device=dev)
@@ -709,7 +718,8 @@ def moe_mlp(x, w_gu, w_down, topk_w, topk_ids, expert_offset: int = 0,
     src = torch.empty(max(n, 1), dtype=torch.int32, device=dev)
     _native_call("dli_moe_align", _p(offsets), _p(pos), _p(src), _p(topk_ids), n, k,
                  expert_offset, E_local, _st())
-    act = torch.empty(max(n, 1), F2 // 2, dtype=x.dtype, device=dev)
+    epi_up = act
+    act = torch.empty(max(n, 1), Fa, dtype=x.dtype, device=dev)
     if n >= _MOE_PREFILL_ROWS * E_local and not torch.cuda.is_current_stream_capturing():
         # prefill-sized expert GEMMs (thousands of rows per expert) are compute-bound: a
         # grouped 256x256 kernel (G.MOE_PREFILL_TILE: the two-barrier 4-wave tile, grid.z =
@@ -724,16 +734,18 @@ def moe_mlp(x, w_gu, w_down, topk_w, topk_ids, expert_offset: int = 0,
         y = torch.empty(max(n, 1), D, dtype=x.dtype, device=dev)
         if rows_max > 0:
             p8 = G.GemmPlan("dli", G.MOE_PREFILL_TILE, 1)
-            _gemm_native(xp, w_gu, "silu_mul", out=act, groups=E_local, group_off=offsets,
-                         rows_per_group=rows_max, plan=p8)
+            # the exact-GELU epilogue lives on the 8-phase 256x256 tile
+            p_up = p8 if G.tile_ok(p8.tile, epi_up) else G.GemmPlan("dli", 22, 1)
+            _gemm_native(xp, w_gu, epi_up, out=act, groups=E_local, group_off=offsets,
+                         rows_per_group=rows_max, plan=p_up)
             _gemm_native(act, w_down, "none", out=y, groups=E_local, group_off=offsets,
                          rows_per_group=rows_max, plan=p8)
         out = torch.empty_like(x)
         _native_call("dli_moe_combine", _p(out), _p(y), _p(topk_w), _p(pos), T, k, D, _st())
         return out
     rows = plan_rows if plan_rows is not None else n
-    p_gu = G.grouped_plan(rows, F2, D, "silu_mul", E_local)
-    if p_gu.splits == 1 and p_gu.tile in G.GATHER_TILES and x.is_contiguous():
+    p_gu = G.grouped_plan(rows, F2, D, epi_up, E_local)
+    if gated and p_gu.splits == 1 and p_gu.tile in G.GATHER_TILES and x.is_contiguous():
         # the gate/up GEMM reads the token rows in place through the permutation (no gathered
         # copy of them: dli_gemm_grouped_gather, the generic tile family)
         _native_call("dli_gemm_grouped_gather", _p(x), x.stride(0), _p(w_gu), w_gu.stride(-2),
@@ -744,15 +756,15 @@ def moe_mlp(x, w_gu, w_down, topk_w, topk_ids, expert_offset: int = 0,
         xp = torch.empty(max(n, 1), D, dtype=x.dtype, device=dev)
         _native_call("dli_moe_gather", _p(xp), _p(x), _p(src), n, D, _p(offsets[E_local:]),
                      _st())
-        _gemm_native(xp, w_gu, "silu_mul", out=act, groups=E_local, group_off=offsets,
+        _gemm_native(xp, w_gu, epi_up, out=act, groups=E_local, group_off=offsets,
                      rows_per_group=n, plan=p_gu)
-    p_dn = G.grouped_plan(rows, D, F2 // 2, "none", E_local)
+    p_dn = G.grouped_plan(rows, D, Fa, "none", E_local)
     if moe_slab_plan(p_dn):
         if defer_combine:
             # the down projection's slabs; the combine runs with the next layer's add + norm
             ws = G.workspace(dev, p_dn.splits * max(n, 1) * D * 2)
             _native_call("dli_gemm", _p(act), act.stride(0), _p(w_down), w_down.stride(-2),
-                         None, D, n, D, F2 // 2, G.EPI["slab16"], p_dn.tile, p_dn.splits, None,
+                         None, D, n, D, Fa, G.EPI["slab16"], p_dn.tile, p_dn.splits, None,
                          _p(ws), _p(offsets), E_local, _st())
             return MoEPending(ws, p_dn.splits, n, topk_w, pos, (T, D), x.dtype, dev)
         out = torch.empty_like(x)

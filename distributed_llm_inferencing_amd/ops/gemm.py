@@ -88,6 +88,8 @@ def tile_ok(tile: int, epi: str) -> bool:
     which must therefore be a multiple of 32."""
     if epi == "res":
         return tile in GEMV_RES_TILES
+    if epi == "gelu_erf" and tile in (34, 41, 45, 55):
+        return False            # the 4-wave families are built without the exact-GELU epilogue
     if tile in (29, 58, 59):
         return epi == "silu_mul"
     if tile in GEMV_TILES:
@@ -103,7 +105,7 @@ def tile_ok(tile: int, epi: str) -> bool:
 # "splitk": a plain GEMM whose fp32 partial slabs feed a fused reduce (ops.linear_add_rmsnorm,
 # ops.linear_rope_cache); planned/tuned separately (a non-split winner runs unfused).
 EPI = {"none": 0, "f32": 1, "silu_mul": 2, "bias_gelu": 3, "bias": 4, "splitk": 0,
-       "slab16": 5}
+       "slab16": 5, "gelu_erf": 6}
 # tiles whose slab-only split-K call can store fp16 partials (EPI "slab16": the generic tile
 # family and the 8-phase kernels); the fused consumers then read half the bytes. The
 # weight-streaming GEMVs and the 4-wave family keep fp32 slabs.
