@@ -315,5 +315,5 @@ int gemm_4w_set_slab_store(int mode);
     case EPI_SILU: return FN<EPI_SILU>(tile_cfg, DLI_GEMM_PASS);                   \
     case EPI_BIAS_GELU: return FN<EPI_BIAS_GELU>(tile_cfg, DLI_GEMM_PASS);         \
     case EPI_BIAS: return FN<EPI_BIAS>(tile_cfg, DLI_GEMM_PASS);                   \
-    default: return (int)hipErrorInvalidValue;                                     \
+    default: return DLI_NOT_MINE; /* another family may build this epilogue */     \
   }

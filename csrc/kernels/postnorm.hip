@@ -30,6 +30,27 @@ template <typename S> __device__ __forceinline__ void stf(S* p, float v);
 template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 
+// four consecutive elements (16-byte aligned fp32, 8-byte aligned bf16)
+template <typename S> __device__ __forceinline__ f32x4 ld4(const S* p);
+template <> __device__ __forceinline__ f32x4 ld4<float>(const float* p) {
+  return *reinterpret_cast<const f32x4*>(p);
+}
+template <> __device__ __forceinline__ f32x4 ld4<u16>(const u16* p) {
+  const uint2 b = *reinterpret_cast<const uint2*>(p);
+  return f32x4{__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u),
+               __uint_as_float(b.y << 16), __uint_as_float(b.y & 0xffff0000u)};
+}
+template <typename S> __device__ __forceinline__ void st4(S* p, f32x4 v);
+template <> __device__ __forceinline__ void st4<float>(float* p, f32x4 v) {
+  *reinterpret_cast<f32x4*>(p) = v;
+}
+template <> __device__ __forceinline__ void st4<u16>(u16* p, f32x4 v) {
+  uint2 pk;
+  pk.x = pack2bf(v[0], v[1]);
+  pk.y = pack2bf(v[2], v[3]);
+  *reinterpret_cast<uint2*>(p) = pk;
+}
+
 // Grid: one workgroup per sequence. Every row's predecessor is read before the slot is
 // overwritten (the barrier), so a one-token portion sees the token of the step before.
 __global__ void __launch_bounds__(256) prev_tokens_kernel(
@@ -80,13 +101,38 @@ template <typename S>
 __global__ void __launch_bounds__(256) postnorm_kernel(
     float* __restrict__ x, const float* __restrict__ y, int ldy, float keep,
     const S* __restrict__ w, const S* __restrict__ b, S* __restrict__ h, int dim, float eps,
-    const long* __restrict__ rows_idx) {
+    const long* __restrict__ rows_idx, bool vec4) {
   extern __shared__ __attribute__((aligned(16))) float row[];   // dim floats + 16 reduction slots
   float* red = row + dim;
   const int r = blockIdx.x;
   const long src = rows_idx ? rows_idx[r] : r;
   float* xr = x + src * dim;
   float s = 0.f;
+  if (vec4) {                                    // 16-byte loads and stores of the rows
+    for (int c = threadIdx.x * 4; c < dim; c += blockDim.x * 4) {
+      f32x4 v = *reinterpret_cast<const f32x4*>(xr + c);
+      if (rows_idx == nullptr) {
+        v *= keep;
+        if (y != nullptr) v += *reinterpret_cast<const f32x4*>(y + (long)r * ldy + c);
+      }
+      *reinterpret_cast<f32x4*>(row + c) = v;
+      s += (v[0] + v[1]) + (v[2] + v[3]);
+    }
+    const float mean = block_sum(s, red) / (float)dim;
+    float q = 0.f;
+    for (int c = threadIdx.x * 4; c < dim; c += blockDim.x * 4) {
+      const f32x4 d = *reinterpret_cast<const f32x4*>(row + c) - mean;
+      q += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
+    }
+    const float rs = 1.f / sqrtf(block_sum(q, red) / (float)dim + eps);
+    for (int c = threadIdx.x * 4; c < dim; c += blockDim.x * 4) {
+      const f32x4 v = (*reinterpret_cast<const f32x4*>(row + c) - mean) * rs * ld4(w + c) +
+                      ld4(b + c);
+      if (rows_idx == nullptr) *reinterpret_cast<f32x4*>(xr + c) = v;
+      st4(h + (long)r * dim + c, v);
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < dim; c += blockDim.x) {
     float v = xr[c];
     if (rows_idx == nullptr) {
@@ -111,11 +157,25 @@ __global__ void __launch_bounds__(256) postnorm_kernel(
 template <typename S>
 __global__ void __launch_bounds__(256) add_rmsnormed_kernel(
     float* __restrict__ x, const float* __restrict__ y, int ldy, const S* __restrict__ w,
-    S* __restrict__ h, int dim, float eps) {
+    S* __restrict__ h, int dim, float eps, bool vec4) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const float* yr = y + (long)r * ldy;
   float s = 0.f;
+  if (vec4) {
+    for (int c = threadIdx.x * 4; c < dim; c += blockDim.x * 4) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(yr + c);
+      s += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+    }
+    const float rs = 1.f / sqrtf(block_sum(s, red) / (float)dim + eps);
+    for (int c = threadIdx.x * 4; c < dim; c += blockDim.x * 4) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(x + (long)r * dim + c) +
+                      *reinterpret_cast<const f32x4*>(yr + c) * rs * ld4(w + c);
+      *reinterpret_cast<f32x4*>(x + (long)r * dim + c) = v;
+      st4(h + (long)r * dim + c, v);
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < dim; c += blockDim.x) { const float v = yr[c]; s += v * v; }
   const float rs = 1.f / sqrtf(block_sum(s, red) / (float)dim + eps);
   for (int c = threadIdx.x; c < dim; c += blockDim.x) {
@@ -340,13 +400,15 @@ extern "C" int dli_postnorm(float* x, const float* y, int ldy, float keep, const
   const size_t sh = (size_t)(dim + 16) * 4;
   if (dim < 1 || sh > 60000 || w == nullptr || b == nullptr || h == nullptr)
     return (int)hipErrorInvalidValue;
+  const bool vec4 = dim % 4 == 0 && ldy % 4 == 0 &&
+                    (((uintptr_t)x | (uintptr_t)y | (uintptr_t)w | (uintptr_t)b | (uintptr_t)h) & 15) == 0;
   DT_SWITCH(dt,
             (postnorm_kernel<u16><<<rows, 256, sh, st>>>(x, y, ldy, keep, (const u16*)w,
                                                          (const u16*)b, (u16*)h, dim, eps,
-                                                         rows_idx)),
+                                                         rows_idx, vec4)),
             (postnorm_kernel<float><<<rows, 256, sh, st>>>(x, y, ldy, keep, (const float*)w,
                                                            (const float*)b, (float*)h, dim, eps,
-                                                           rows_idx)));
+                                                           rows_idx, vec4)));
   DLI_RETURN_LAUNCH();
 }
 
@@ -354,11 +416,13 @@ extern "C" int dli_add_rmsnormed(float* x, const float* y, int ldy, const void* 
                                  int rows, int dim, float eps, int dt, hipStream_t st) {
   if (rows <= 0) return 0;
   if (dim < 1) return (int)hipErrorInvalidValue;
+  const bool vec4 = dim % 4 == 0 && ldy % 4 == 0 &&
+                    (((uintptr_t)x | (uintptr_t)y | (uintptr_t)w | (uintptr_t)h) & 15) == 0;
   DT_SWITCH(dt,
             (add_rmsnormed_kernel<u16><<<rows, 256, 0, st>>>(x, y, ldy, (const u16*)w, (u16*)h,
-                                                             dim, eps)),
+                                                             dim, eps, vec4)),
             (add_rmsnormed_kernel<float><<<rows, 256, 0, st>>>(x, y, ldy, (const float*)w,
-                                                               (float*)h, dim, eps)));
+                                                               (float*)h, dim, eps, vec4)));
   DLI_RETURN_LAUNCH();
 }
 

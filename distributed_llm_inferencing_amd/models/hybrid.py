@@ -86,7 +86,7 @@ class HybridLM(TransformerLM):
             raise ValueError("hybrid models attend through the paged cache: the step carries "
                              "no block tables")
         return StepView(cu, mx, b.positions, b.slot_mapping, b.block_tables, block_size,
-                        b.state_slots)
+                        b.state_slots, b.max_context if b.max_context > 0 else 1 << 30)
 
     def _all_rows(self, n: int) -> torch.Tensor:
         r = self._rows.get(n)

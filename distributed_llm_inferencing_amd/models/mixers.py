@@ -32,6 +32,7 @@ class StepView:
     block_tables: torch.Tensor      # [S, W] int32
     block_size: int
     state_slots: Optional[torch.Tensor]   # [S] int32 recurrent-state slot (-1: padding row)
+    max_context: int = 1 << 30      # no position of this step is at or beyond this
 
 
 def derive_constants(spec: LayerSpec, lp: dict, device) -> None:
@@ -109,9 +110,12 @@ def latent_attention_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, 
         q_nope, q_full = H.mla_prepare(proj, lp["c_norm"], eps, Hh, d, dr, r, spec.rot_dims,
                                        lp["inv_freq"], step.positions, step.slot_mapping, c)
     H.head_linear(q_nope, lp["w_ukT"], q_full)               # q_full[:, h, :r] = W_uk,h^T q_h
+    # a window no shorter than the step's longest context masks nothing: the tight bound lets
+    # the kernel size its slot table and key splits for the keys that exist
+    win = min(spec.window, max(1, step.max_context))
     ol = H.window_attention(q_full.view(T, Hh * (r + dr)), c, c, r + dr, r, Hh, 1,
                             step.cu_seqlens, step.max_seqlen, step.positions,
-                            step.block_tables, step.block_size, spec.window, spec.scale)
+                            step.block_tables, step.block_size, win, spec.scale)
     if gates is not None:                   # one sigmoid gate per head, on the fp32 expansion
         o32 = torch.empty(T, Hh, dv, dtype=torch.float32, device=h.device)
         H.head_linear(ol.view(T, Hh, r), lp["w_uv"], o32)

@@ -58,6 +58,14 @@ def config(layers, width=40, vocab=80, eps=1e-5, alpha=2.5, bigram=(53, 11, 3), 
     return c
 
 
+def without_routing(c):
+    c = copy.deepcopy(c)
+    for L in c["layers"]:
+        if L["mlp"] and L["mlp"]["kind"] == "moe":
+            L["mlp"] = dense(16)
+    return c
+
+
 FULL = config([gla(mlp=dense()), latent(mlp=moe()), latent(kv_from=1, mlp=moe(top=3, shared=0)),
                gla(heads=3, dim=4, vdim=4, tau=2.0, mlp=moe(experts=3, top=1)),
                latent(heads=2, dim=16, rot=8, vdim=4, kv_rank=8, q_rank=5, mlp=None),
@@ -90,15 +98,17 @@ def ref(tokens, c, w):
     return Ref(O.forward(c, w, tokens).numpy(), O.route_margins(c, w, tokens))
 
 
-def close(got, want, dtype, what=""):
+def close(got, want, dtype, what="", slack=1.0):
     """Row error as a logit comparison sees it: mean removed, relative to the spread. In bf16
     a position whose routing was a close call (the rounded input may choose another expert,
-    which with one expert per token swaps the whole feed-forward output) only has to stay
-    bounded; every other position, and fp32 everywhere, is held to the strict bound."""
+    which with one expert per token swaps the whole feed-forward output) and the positions
+    after it (they read its state and keys) only have to stay bounded; every position before,
+    every position of a model without routing, and fp32 everywhere, is held to the strict
+    bound."""
     loose = None
     if isinstance(want, Ref):
         if dtype == torch.bfloat16:
-            loose = want.margins < 0.02
+            loose = np.maximum.accumulate(want.margins < 0.02)
         want = want.logits
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     d = got - want
@@ -108,7 +118,8 @@ def close(got, want, dtype, what=""):
         assert err[loose].max() < 2.5, what
         err = err[~loose]
     if err.size:
-        assert err.max() < tol(dtype), f"{what}: error {err.max():.3g} at row {int(err.argmax())}"
+        assert err.max() < slack * tol(dtype), \
+            f"{what}: error {err.max():.3g} at row {int(err.argmax())}"
 
 
 def replay(eng, tokens, cuts, rid="a"):
@@ -348,7 +359,9 @@ def test_layer_trace_matches_the_oracle(device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-def test_prefill_equals_decode_equals_portions(device, dtype):
+@pytest.mark.parametrize("routed", [True, False])
+def test_prefill_equals_decode_equals_portions(device, dtype, routed):
+    FULL = globals()["FULL"] if routed else without_routing(globals()["FULL"])
     w = O.random_weights(FULL, 1)
     t = toks(45, FULL["vocab"], 3)
     want = ref(t, FULL, w)
@@ -449,14 +462,17 @@ def test_far_keys_and_page_borders_stand_out(far, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-def test_first_tokens_and_long_decode(device, dtype):
+@pytest.mark.parametrize("routed", [True, False])
+def test_first_tokens_and_long_decode(device, dtype, routed):
+    FULL = globals()["FULL"] if routed else without_routing(globals()["FULL"])
     w = O.random_weights(FULL, 6)
     t = toks(150, FULL["vocab"], 8)
     want = ref(t, FULL, w)
     eng = engine(FULL, w, device, dtype)
     got = replay(eng, t, [1, 1, 1, 2] + [1] * 145)
     close(got[:6], want[:6], dtype, "first tokens")
-    close(got, want, dtype, "long decode")
+    # 150 steps of six layers: bf16 rounding of the activations adds up along the states
+    close(got, want, dtype, "long decode", slack=1.0 if dtype == torch.float32 else 2.0)
     # the same slot and pages again, starting from a stale state
     t2 = toks(12, FULL["vocab"], 9)
     close(replay(eng, t2, [1] * 12), ref(t2, FULL, w), dtype, "reused")
