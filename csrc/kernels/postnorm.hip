@@ -205,12 +205,23 @@ __global__ void __launch_bounds__(256) side_gate_kernel(
 template <typename S>
 __global__ void __launch_bounds__(256) rmsnorm_cols_kernel(
     S* __restrict__ out, const float* __restrict__ src, int lds, const S* __restrict__ w, int T,
-    int n, float eps) {
+    int n, float eps, bool vec4) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (t >= T) return;
   const float* r = src + (long)t * lds;
   float s = 0.f;
+  if (vec4) {                                   // 16-byte loads, 4 columns a lane
+    for (int c = lane * 4; c < n; c += 256) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(r + c);
+      s += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+    }
+    s = wave_sum(s);
+    const float rs = 1.f / sqrtf(s / (float)n + eps);
+    for (int c = lane * 4; c < n; c += 256)
+      st4(out + (long)t * n + c, *reinterpret_cast<const f32x4*>(r + c) * rs * ld4(w + c));
+    return;
+  }
   for (int c = lane; c < n; c += 64) { const float v = r[c]; s += v * v; }
   s = wave_sum(s);
   const float rs = 1.f / sqrtf(s / (float)n + eps);
@@ -221,16 +232,15 @@ __global__ void __launch_bounds__(256) rmsnorm_cols_kernel(
 // i < rot_dims/2 pairs with i + rot_dims/2, else pairs are (2i, 2i+1). The pair (u, v) at angle
 // a becomes (u cos a - v sin a, v cos a + u sin a); the angle position * frequency is formed in
 // double and rounded once.
+// `cs` / `sn` [rot_dims / 2]: this token's cosines and sines (LDS).
 __device__ __forceinline__ float rotate_elem(const float* v, int c, int rot_dims, bool half,
-                                             double pos, const double* inv_freq) {
+                                             const float* cs, const float* sn) {
   if (c >= rot_dims) return v[c];
   const int hd = rot_dims >> 1;
   const int i = half ? (c < hd ? c : c - hd) : (c >> 1);
   const bool second = half ? c >= hd : (c & 1);
   const int partner = half ? (second ? c - hd : c + hd) : (c ^ 1);
-  const double a = pos * inv_freq[i];
-  const float cs = (float)cos(a), sn = (float)sin(a);
-  return second ? v[c] * cs + v[partner] * sn : v[c] * cs - v[partner] * sn;
+  return second ? v[c] * cs[i] + v[partner] * sn[i] : v[c] * cs[i] - v[partner] * sn[i];
 }
 
 // Grid: one workgroup per token. qproj row (fp32): H heads of [d unrotated | dr rotated].
@@ -245,8 +255,17 @@ __global__ void __launch_bounds__(256) latent_prepare_kernel(
     const int* __restrict__ slots, S* __restrict__ q_nope, S* __restrict__ q_full,
     S* __restrict__ cache, bool half) {
   __shared__ float red[16];
+  extern __shared__ float trig[];               // [rot_dims / 2] cosines, then sines
+  float* cs = trig;
+  float* sn = trig + (rot_dims >> 1);
   const int t = blockIdx.x;
   const double pos = (double)positions[t];
+  for (int i = threadIdx.x; i < (rot_dims >> 1); i += blockDim.x) {
+    const double a = pos * inv_freq[i];         // the angle in double, rounded once
+    cs[i] = (float)cos(a);
+    sn[i] = (float)sin(a);
+  }
+  __syncthreads();
   if (kvproj != nullptr) {
     const float* dkv = kvproj + (long)t * ldkv;
     const int slot = slots[t];
@@ -258,7 +277,7 @@ __global__ void __launch_bounds__(256) latent_prepare_kernel(
       S* cr = cache + (long)slot * (r + dr);
       for (int c = threadIdx.x; c < r; c += blockDim.x) stf(cr + c, dkv[c] * rs * ldf(cw + c));
       for (int c = threadIdx.x; c < dr; c += blockDim.x)
-        stf(cr + r + c, rotate_elem(dkv + r, c, rot_dims, half, pos, inv_freq));
+        stf(cr + r + c, rotate_elem(dkv + r, c, rot_dims, half, cs, sn));
     }
   }
   const float* row = qproj + (long)t * ldq;
@@ -268,7 +287,7 @@ __global__ void __launch_bounds__(256) latent_prepare_kernel(
       stf(q_nope + ((long)t * H + h) * d + c, row[i]);
     } else {
       stf(q_full + ((long)t * H + h) * (r + dr) + r + (c - d),
-          rotate_elem(row + h * (d + dr) + d, c - d, rot_dims, half, pos, inv_freq));
+          rotate_elem(row + h * (d + dr) + d, c - d, rot_dims, half, cs, sn));
     }
   }
 }
@@ -446,11 +465,13 @@ extern "C" int dli_rmsnorm_cols(void* out, const float* src, int lds, const void
   if (T <= 0) return 0;
   if (n < 1) return (int)hipErrorInvalidValue;
   const int nb = (T + 3) / 4;
+  const bool vec4 = n % 4 == 0 && lds % 4 == 0 &&
+                    (((uintptr_t)out | (uintptr_t)src | (uintptr_t)w) & 15) == 0;
   DT_SWITCH(dt,
             (rmsnorm_cols_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, src, lds, (const u16*)w, T,
-                                                          n, eps)),
+                                                          n, eps, vec4)),
             (rmsnorm_cols_kernel<float><<<nb, 256, 0, st>>>((float*)out, src, lds,
-                                                            (const float*)w, T, n, eps)));
+                                                            (const float*)w, T, n, eps, vec4)));
   DLI_RETURN_LAUNCH();
 }
 
@@ -460,14 +481,15 @@ extern "C" int dli_latent_prepare(const float* qproj, int ldq, const float* kvpr
                                   const int* slots, void* q_nope, void* q_full, void* cache,
                                   int half, int dt, hipStream_t st) {
   if (T <= 0) return 0;
-  if (rot_dims > dr || (rot_dims & 1) || H < 1 || d < 1 || r < 1) return (int)hipErrorInvalidValue;
+  if (rot_dims > dr || (rot_dims & 1) || rot_dims > 8192 || H < 1 || d < 1 || r < 1)
+    return (int)hipErrorInvalidValue;
   if (kvproj != nullptr && (cw == nullptr || cache == nullptr || slots == nullptr))
     return (int)hipErrorInvalidValue;
   DT_SWITCH(dt,
-            (latent_prepare_kernel<u16><<<T, 256, 0, st>>>(
+            (latent_prepare_kernel<u16><<<T, 256, (size_t)rot_dims * 4, st>>>(
                 qproj, ldq, kvproj, ldkv, (const u16*)cw, eps, H, d, dr, r, rot_dims, inv_freq,
                 positions, slots, (u16*)q_nope, (u16*)q_full, (u16*)cache, half != 0)),
-            (latent_prepare_kernel<float><<<T, 256, 0, st>>>(
+            (latent_prepare_kernel<float><<<T, 256, (size_t)rot_dims * 4, st>>>(
                 qproj, ldq, kvproj, ldkv, (const float*)cw, eps, H, d, dr, r, rot_dims, inv_freq,
                 positions, slots, (float*)q_nope, (float*)q_full, (float*)cache, half != 0)));
   DLI_RETURN_LAUNCH();

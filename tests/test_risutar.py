@@ -213,7 +213,7 @@ def test_norm_after_the_sum_and_normed_side_input(device, dtype):
 
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("H_,d,dv,tau", [(2, 8, 12, 6.0), (3, 5, 3, 1.0), (1, 16, 64, 16.0),
-                                         (2, 32, 16, 3.0), (1, 64, 70, 2.0)])
+                                         (2, 32, 16, 3.0), (1, 64, 70, 2.0), (1, 128, 32, 9.0)])
 def test_gated_linear_attention_and_its_state(device, dtype, H_, d, dv, tau):
     """The recurrence over portions and single tokens of two interleaved sequences whose
     slots held stale states, against the oracle run over each whole sequence."""
@@ -418,6 +418,11 @@ def test_other_sizes_and_degenerate_values(device, dtype):
                width=28, vocab=40, alpha=0.5, bigram=None, side=0),
         config([latent(mlp=dense()), gla(mlp=None)], width=64, vocab=50, eps=1e-2, alpha=7.0,
                bigram=(1, 3, 2), side=13),
+        # nothing a multiple of 4: no kernel may take a vector path it is not aligned for
+        config([latent(heads=3, dim=5, rot=2, vdim=3, kv_rank=7, q_rank=5, mlp=moe(ff=5, experts=3, top=2, shared=7)),
+                gla(heads=3, dim=5, vdim=7, tau=3.0, mlp=dense(9)),
+                latent(heads=1, dim=3, rot=2, vdim=9, kv_rank=7, q_rank=3, kv_from=0, mlp=None)],
+               width=30, vocab=33, alpha=1.5, bigram=(5, 2, 9), side=3),
     ]
     for n, c in enumerate(cs):
         w = O.random_weights(c, 20 + n, decay_rank=1 + 3 * n)
