@@ -95,8 +95,9 @@ def _design_sweep(cfgs, a, V):
             del eng
             torch.cuda.empty_cache()
         for (B, C) in a.design_decode:
-            # the decoded tokens stay inside the block that ends at C: the block mask's worst
-            # case (a nearly full block of keys), not the few keys after a block edge
+            # the decoded tokens stay inside the block of C positions that ends at C: for a
+            # block mask its worst case (a nearly full block of keys, not the few keys after
+            # a block edge); an unmasked design simply decodes at contexts just below C
             n_new = 33
             C = max(1, C - n_new - 7)
             eng = LLMEngine(cfg, device="cuda:0", max_batch=B, max_model_len=C + n_new + 16,
@@ -178,7 +179,7 @@ def run_design_risutar(a):
                experts=E, top=top, shared_ff=3072)
 
     def gla():
-        return LayerSpec("gla", heads=Hh, dim=hd, vdim=hd, tau=16.0, decay_rank=16, **moe)
+        return LayerSpec("gla", heads=Hh, dim=hd, vdim=hd, tau=8.0, decay_rank=32, **moe)
 
     def latent(kv_from=-1):
         return LayerSpec("latent_attention", heads=Hh, kv_heads=1, dim=hd, vdim=hd,
@@ -186,8 +187,8 @@ def run_design_risutar(a):
                          rot_dims=64, q_rank=1536, head_gate=True, rot_half=True,
                          kv_from=kv_from, **moe)
     hyb = hybrid_config("risutar-bench", D, V, (gla(), latent(), latent(1), gla()),
-                        arch="risutar", max_position=1 << 15, norm_eps=1e-5, postln_alpha=3.0,
-                        bigram=(65521, 127, 7), side_dim=16)
+                        arch="risutar", max_position=1 << 15, norm_eps=1e-6, postln_alpha=2.0,
+                        bigram=(65521, 31, 17), side_dim=32)
     mix = replace(get_config("mixtral-8x7b"), name="mixtral-bench", hidden_size=D, num_layers=4,
                   num_heads=Hh, num_kv_heads=G, head_dim=hd, intermediate_size=Fw, vocab_size=V,
                   num_experts=E, top_k_experts=top, max_position=1 << 15)
@@ -197,7 +198,7 @@ def run_design_risutar(a):
                       "dtype": "bf16", "data": "synthetic prompts, random-init weights",
                       "config": {"width": D, "expert_ff": Fw * 3 // 2, "layers": 4, "heads": Hh,
                                  "head_dim": hd, "kv_rank": 512, "q_rank": 1536, "rot_dim": 64,
-                                 "experts": E, "top": top, "shared_ff": 3072, "side_dim": 16,
+                                 "experts": E, "top": top, "shared_ff": 3072, "side_dim": 32,
                                  "bigram_buckets": 65521},
                       "results": out}), flush=True)
 

@@ -328,7 +328,7 @@ RISUTAR_TINY = hybrid_config(
         LayerSpec("latent_attention", **_RISUTAR_LATENT, kv_from=0,
                   **_risutar_moe(ff=64, experts=4, top=1)),
         LayerSpec("gla", heads=4, dim=16, vdim=16, tau=4.0, decay_rank=4, ff=0)),
-    norm_eps=1e-5, postln_alpha=2.0, bigram=(251, 31, 5), side_dim=8)
+    norm_eps=1e-6, postln_alpha=2.0, bigram=(251, 31, 5), side_dim=8)
 
 _REGISTRY = {c.name: c for c in
              (GPT2, LLAMA3_8B, LLAMA3_70B, MIXTRAL_8X7B, LLAMA_TINY, LLAMA_TINY128,

@@ -767,7 +767,7 @@ def gla(proj, z, a_bias, tau, norm_w, eps, state, slots, cu_seqlens, positions, 
 
 def logit_router(h, w_router, bias, top):
     """Router logits h @ w_router^T + bias in fp32; the ``top`` largest are chosen (lowest
-    index on ties) and weighted by the softmax over the chosen logits only. Returns (weights
+    index on ties) and weighted by a softmax renormalised over those ``top`` logits. Returns (weights
     fp32 [T, top], ids int32 [T, top])."""
     z = h.float() @ w_router.float().t() + bias.float()
     order = torch.sort(z, dim=-1, descending=True, stable=True)

@@ -135,7 +135,7 @@ def expert(sd, pre, h):
 
 
 def route(mlp, sd, pre, h):
-    """(ids [T, top], weights [T, top]): the largest logits, softmax over the chosen only."""
+    """(ids [T, top], weights [T, top]): top-k by logit, weights renormalised among the k."""
     z = h @ f64(sd[pre + "router"]).T + f64(sd[pre + "router.b"])
     top = mlp["router"]["top"]
     val, ids = torch.topk(z, top, dim=-1)

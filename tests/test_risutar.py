@@ -48,7 +48,7 @@ def latent(heads=3, dim=8, rot=4, vdim=10, kv_rank=12, q_rank=14, scale=0.3, bas
     return {"type": "latent_attention", "mixer": mx, "mlp": mlp}
 
 
-def config(layers, width=40, vocab=80, eps=1e-5, alpha=2.5, bigram=(53, 11, 3), side=6):
+def config(layers, width=40, vocab=80, eps=2e-6, alpha=2.5, bigram=(53, 11, 3), side=6):
     c = {"architecture": "Risutar", "width": width, "vocab": vocab, "norm": {"eps": eps},
          "postln_alpha": alpha, "layers": layers}
     if bigram:
@@ -309,7 +309,7 @@ def test_latent_attention_own_and_borrowed_cache(device, dtype, H_, d, dr, dv, r
                                  moe(ff=7, experts=9, top=4, shared=5)],
                          ids=["usual", "top1", "all_experts", "no_shared", "odd_sizes"])
 def test_router_and_experts(device, dtype, mlp):
-    """Biased logits, the largest chosen, softmax over the chosen only, exact-GELU experts,
+    """Biased logits, top-k by logit, weights renormalised among the k, exact-GELU experts,
     the always-on shared expert."""
     from distributed_llm_inferencing_amd.models.mixers import derive_constants, moe_ff
     D, T = 24, 33
@@ -510,7 +510,7 @@ def test_greedy_generation_through_the_engine(device, dtype, graphs):
 def test_config_reader_reads_every_size():
     cfg = config_from_hf(FULL)
     assert cfg.arch == "risutar" and cfg.is_hybrid and cfg.has_state
-    assert (cfg.hidden_size, cfg.vocab_size, cfg.postln_alpha, cfg.norm_eps) == (40, 80, 2.5, 1e-5)
+    assert (cfg.hidden_size, cfg.vocab_size, cfg.postln_alpha, cfg.norm_eps) == (40, 80, 2.5, 2e-6)
     assert cfg.bigram == (53, 11, 3) and cfg.side_dim == 6
     s = cfg.layer_specs
     assert [x.kind for x in s] == ["gla", "latent_attention", "latent_attention", "gla",
