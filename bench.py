@@ -187,7 +187,7 @@ def run_design_risutar(a):
                          rot_dims=64, q_rank=1536, head_gate=True, rot_half=True,
                          kv_from=kv_from, **moe)
     hyb = hybrid_config("risutar-bench", D, V, (gla(), latent(), latent(1), gla()),
-                        arch="risutar", max_position=1 << 15, norm_eps=1e-6, postln_alpha=2.0,
+                        arch="risutar", max_position=1 << 15, norm_eps=1e-6, post_norm=True, postln_alpha=2.0,
                         bigram=(65521, 31, 17), side_dim=32)
     mix = replace(get_config("mixtral-8x7b"), name="mixtral-bench", hidden_size=D, num_layers=4,
                   num_heads=Hh, num_kv_heads=G, head_dim=hd, intermediate_size=Fw, vocab_size=V,

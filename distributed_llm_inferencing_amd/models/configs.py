@@ -108,8 +108,9 @@ class ModelConfig:
     learned_pos: bool = False     # a learned vector per position is added to the embedding
     scalar_norm: bool = False     # every norm's weight is one number (checkpoint layout)
     # post-norm layers (arch "risutar"): x = LayerNorm(postln_alpha * x + sublayer(x)) with
-    # weight and bias, the sublayers reading x itself; 0 = pre-norm residual layers
-    postln_alpha: float = 0.0
+    # weight and bias, the sublayers reading x itself; False = pre-norm residual layers
+    post_norm: bool = False
+    postln_alpha: float = 1.0
     # hashed bigram embedding (buckets, mul_prev, mul_cur): row (prev * mul_prev + cur *
     # mul_cur) mod buckets of a second table is added, row ``buckets`` for a first token
     bigram: tuple = ()
@@ -328,7 +329,7 @@ RISUTAR_TINY = hybrid_config(
         LayerSpec("latent_attention", **_RISUTAR_LATENT, kv_from=0,
                   **_risutar_moe(ff=64, experts=4, top=1)),
         LayerSpec("gla", heads=4, dim=16, vdim=16, tau=4.0, decay_rank=4, ff=0)),
-    norm_eps=1e-6, postln_alpha=2.0, bigram=(251, 31, 5), side_dim=8)
+    norm_eps=1e-6, post_norm=True, postln_alpha=2.0, bigram=(251, 31, 5), side_dim=8)
 
 _REGISTRY = {c.name: c for c in
              (GPT2, LLAMA3_8B, LLAMA3_70B, MIXTRAL_8X7B, LLAMA_TINY, LLAMA_TINY128,

@@ -219,7 +219,7 @@ def risutar_config(c: dict, name: Optional[str] = None) -> ModelConfig:
     bigram = (int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"])) if bg else ()
     return hybrid_config(name or c.get("_name_or_path") or "risutar", int(c["width"]),
                          int(c["vocab"]), specs, norm_eps=float((c.get("norm") or {}).get("eps", 1e-5)),
-                         arch="risutar", postln_alpha=float(c.get("postln_alpha", 1.0)),
+                         arch="risutar", post_norm=True, postln_alpha=float(c.get("postln_alpha", 1.0)),
                          bigram=bigram, side_dim=int((c.get("token_side") or {}).get("dim") or 0))
 
 

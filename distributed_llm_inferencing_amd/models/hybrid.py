@@ -7,7 +7,7 @@ same engine, scheduler, block manager and runner as the transformer families.
     embed (fp32) -> per layer run: x += m * mixer(gnorm(x)); x += m * ff(gnorm(x))
                  -> gnorm -> LM head (fp32 logits) -> sampler
 
-Post-norm designs (``cfg.postln_alpha``; ``risutar``) run
+Post-norm designs (``cfg.post_norm``; ``risutar``) run
 
     embed + hashed bigram (fp32) -> per layer: x = LN(a x + mixer(x)); x = LN(a x + ff(x));
                  x += rmsnorm(side_proj(gelu(side_gate x) * side_embed[token]))
@@ -97,7 +97,7 @@ class HybridLM(TransformerLM):
     # ------------------------------------------------------------------ forward
     def embed(self, b: DeviceBatch, kv_caches=None) -> torch.Tensor:
         cfg, p = self.cfg, self.params
-        if cfg.postln_alpha:
+        if cfg.post_norm:
             # (fp32 stream, its storage-dtype rounding): the first layer's sublayers read both
             prev, bg = None, cfg.bigram or (0, 0, 0)
             if cfg.bigram:
@@ -134,7 +134,7 @@ class HybridLM(TransformerLM):
 
     def forward_layers(self, x: torch.Tensor, b: DeviceBatch, kv_caches) -> torch.Tensor:
         cfg, p = self.cfg, self.params
-        if cfg.postln_alpha:
+        if cfg.post_norm:
             return self._postnorm_layers(x, b, kv_caches)
         eps, groups, m = cfg.norm_eps, cfg.norm_groups, cfg.residual_mult
         step = self._step_view(b, kv_caches.block_size)
@@ -177,7 +177,7 @@ class HybridLM(TransformerLM):
             rows = b.last_token_idx
         else:
             rows = None
-        if cfg.postln_alpha:
+        if cfg.post_norm:
             if rows is None:
                 rows = self._all_rows(hidden.shape[0])
             return H.postnorm(hidden, None, p["final_norm"], p["final_norm_b"], cfg.norm_eps,

@@ -87,7 +87,7 @@ def hybrid_layer_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
                     p + "talk": (H, H), p + "wo": (D, H * dv)})
     else:
         raise ValueError(f"unknown mixer kind '{s.kind}'")
-    if cfg.postln_alpha:
+    if cfg.post_norm:
         out[p + "norm1_b"] = (D,)
         if s.ff:
             out[p + "norm2_b"] = (D,)
@@ -145,7 +145,7 @@ def global_param_shapes(cfg: ModelConfig, first: bool, last: bool) -> Dict[str, 
             s.update({"loop_in": (d, 2 * d), "loop_step": (cfg.loop[2], d)})
         if cfg.learned_pos:
             s["pos_embed"] = (cfg.max_position, d)
-        if cfg.postln_alpha:
+        if cfg.post_norm:
             s["final_norm_b"] = (d,)
         if cfg.bigram:
             s["bigram"] = (cfg.bigram[0] + 1, d)
