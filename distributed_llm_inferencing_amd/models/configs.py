@@ -66,19 +66,42 @@ class LayerSpec:
     rot_half: bool = False    # rotation pairs (i, i + rot_dims/2) instead of (2i, 2i+1)
     tau: float = 1.0          # gla: the decay is sigmoid(z)^(1/tau)
     decay_rank: int = 0       # gla: inner width of the decay's two-step projection
+    decays: tuple = ()        # lightning: the state's decay per head
+    rot_scaling: tuple = ()   # sink_attention: YaRN (factor, original, fast, slow) or ()
+    gate_cap: float = 0.0     # mlstm: soft cap of the gate pre-activations
+    left: Optional["LayerSpec"] = None     # parallel: the attention side
+    right: Optional["LayerSpec"] = None    # parallel: the recurrent side
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    router_groups: int = 1    # group_score router: equal groups of neighbouring experts
+    router_keep: int = 1      # ... of which the best this many may be chosen from
+    router_scale: float = 1.0     # ... and the chosen scores are multiplied by this
+    act_limit: float = 0.0    # clamp_swish experts: the clamp
 
     @property
     def has_state(self) -> bool:
         """The layer keeps something per sequence besides cache rows: a recurrent state, or
         the previous token's mixer input."""
-        return self.kind in ("hgrn2", "gla") or self.shift
+        return self.kind in ("hgrn2", "gla", "lightning", "parallel", "mlstm") or self.shift
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "LayerSpec":
+        kw = dict(d)
+        for side in ("left", "right"):
+            if isinstance(kw.get(side), dict):
+                kw[side] = cls.from_dict(kw[side])
+        for k in ("decays", "rot_scaling"):
+            if k in kw:
+                kw[k] = tuple(kw[k] or ())
+        return cls(**kw)
 
 
 @dataclass(frozen=True)
 class ModelConfig:
     name: str
     arch: str                 # "llama" (llama / mixtral family), "gpt2", or a hybrid
-                              # (layer-list) design: "buborax", "pulunex", "risutar"
+                              # (layer-list) design: "buborax", "pulunex", "risutar",
+                              # "lapunex"
     hidden_size: int
     num_layers: int
     num_heads: int
@@ -116,6 +139,14 @@ class ModelConfig:
     bigram: tuple = ()
     # per-layer token input: width of each layer's slice of a second embedding table
     side_dim: int = 0
+    # hyper-connections: this many copies of the residual stream (0: one plain stream); each
+    # sublayer reads a learned combination of them and writes back through a learned mix
+    streams: int = 0
+    # norm weights are stored as offsets from this value (1.0: weights around zero)
+    norm_offset: float = 0.0
+    # a loop pass starts with x = W_in [x ; x0] + step[pass]; False: passes follow each other
+    # with nothing in between
+    loop_entry: bool = True
 
     @property
     def is_hybrid(self) -> bool:
@@ -131,7 +162,7 @@ class ModelConfig:
         start, stop, times = self.loop
         runs = [(i, -1, False) for i in range(start)]
         for t in range(times):
-            runs += [(i, t, i == start) for i in range(start, stop)]
+            runs += [(i, t, i == start and self.loop_entry) for i in range(start, stop)]
         return runs + [(i, -1, False) for i in range(stop, n)]
 
     @property
@@ -204,6 +235,8 @@ class ModelConfig:
             return 0 if s.kv_from >= 0 else s.kv_rank + s.rot_dim
         if s.kind == "talk_attention":
             return 0 if s.kv_from >= 0 else s.kv_heads * (s.dim + s.vdim)
+        if s.kind == "parallel":
+            return s.left.kv_heads * (s.left.dim + s.left.vdim)
         return 0
 
     def to_dict(self) -> dict:
@@ -214,7 +247,7 @@ class ModelConfig:
         fields = cls.__dataclass_fields__.keys()
         kw = {k: v for k, v in d.items() if k in fields}
         if kw.get("layer_specs"):
-            kw["layer_specs"] = tuple(s if isinstance(s, LayerSpec) else LayerSpec(**s)
+            kw["layer_specs"] = tuple(s if isinstance(s, LayerSpec) else LayerSpec.from_dict(s)
                                       for s in kw["layer_specs"])
         if "loop" in kw:
             kw["loop"] = tuple(kw["loop"] or ())
@@ -331,10 +364,33 @@ RISUTAR_TINY = hybrid_config(
         LayerSpec("gla", heads=4, dim=16, vdim=16, tau=4.0, decay_rank=4, ff=0)),
     norm_eps=1e-6, post_norm=True, postln_alpha=2.0, bigram=(251, 31, 5), side_dim=8)
 
+def _lapunex_moe(**kw) -> dict:
+    return dict(ff_kind="moe", router="group_score", expert_act="clamp_swish", **kw)
+
+
+# Lapunex at test size: hyper-connected streams, lightning layers, a parallel attention +
+# matrix-memory layer, dense and routed feed-forwards, a loop without an entry projection
+LAPUNEX_TINY = hybrid_config(
+    "lapunex-tiny", width=128, vocab=384, arch="lapunex",
+    layer_specs=(
+        LayerSpec("lightning", heads=2, dim=32, vdim=16, decays=(0.7, 0.97), ff=192,
+                  ff_kind="gated_silu"),
+        LayerSpec("parallel", heads=4, dim=32, vdim=32,
+                  left=LayerSpec("sink_attention", heads=4, kv_heads=2, dim=32, vdim=16,
+                                 scale=0.2, rot_dims=8, rot_base=1000.0,
+                                 rot_scaling=(4.0, 64.0, 16.0, 1.0)),
+                  right=LayerSpec("mlstm", heads=2, dim=16, vdim=32, gate_cap=10.0),
+                  left_scale=0.7, right_scale=0.6,
+                  **_lapunex_moe(ff=48, experts=6, top=2, router_groups=3, router_keep=2,
+                                 router_scale=1.2, act_limit=2.0)),
+        LayerSpec("lightning", heads=4, dim=16, vdim=32, decays=(0.5, 0.8, 0.9, 0.99), ff=0)),
+    loop=(0, 2, 2), norm_eps=1e-5, embed_scale=6.0, streams=2, norm_offset=1.0,
+    loop_entry=False)
+
 _REGISTRY = {c.name: c for c in
              (GPT2, LLAMA3_8B, LLAMA3_70B, MIXTRAL_8X7B, LLAMA_TINY, LLAMA_TINY128,
               LLAMA_TINY8, MIXTRAL_TINY, MIXTRAL_TINY8E, GPT2_TINY, BUBORAX_TINY, PULUNEX_TINY,
-              RISUTAR_TINY)}
+              RISUTAR_TINY, LAPUNEX_TINY)}
 
 _ALIASES = {
     "openai-community/gpt2": "gpt2",

@@ -25,8 +25,8 @@ from typing import Dict, Iterable, Iterator, Optional, Tuple
 import torch
 
 from .configs import ModelConfig
-from .weights import (from_buborax_state_dict, from_hf_state_dict, from_pulunex_state_dict,
-                      from_risutar_state_dict)
+from .weights import (from_buborax_state_dict, from_hf_state_dict, from_lapunex_state_dict,
+                      from_pulunex_state_dict, from_risutar_state_dict)
 
 
 def is_hf_dir(d) -> bool:
@@ -59,7 +59,7 @@ def find_hf_dir(root: str, name: str) -> Optional[Path]:
     return None
 
 
-NATIVE_ARCHS = ("Buborax", "Pulunex", "Risutar")
+NATIVE_ARCHS = ("Buborax", "Pulunex", "Risutar", "Lapunex")
 
 
 def buborax_config(c: dict, name: Optional[str] = None) -> ModelConfig:
@@ -223,15 +223,94 @@ def risutar_config(c: dict, name: Optional[str] = None) -> ModelConfig:
                          bigram=bigram, side_dim=int((c.get("token_side") or {}).get("dim") or 0))
 
 
+def lapunex_config(c: dict, name: Optional[str] = None) -> ModelConfig:
+    """A Lapunex ``config.json``: ``width``, ``vocab``, ``norm`` {eps}, ``embedding`` {scale},
+    ``streams`` (optional: hyper-connected copies of the residual stream), ``loop`` {start,
+    stop, times} (optional) and ``layers``, a list of {type, mixer, mlp}: type ``lightning``
+    with mixer {heads, dim, vdim, decay [per head]} or ``parallel`` with mixer {left {heads,
+    kv_heads, dim, vdim, scale, rot {base, dims, scaling {factor, original, fast, slow}}},
+    right {heads, dim, vdim, gate_cap}, left_scale, right_scale}; mlp null, {kind: dense, ff}
+    or {kind: moe, expert {ff, limit}, router {experts, top, scale, groups {count, keep}}}.
+    Every size and constant is read from it."""
+    from .configs import LayerSpec, hybrid_config
+    specs = []
+    for i, L in enumerate(c["layers"]):
+        mx, kind = L["mixer"], L["type"]
+        ff = dict(ff=0)
+        mlp = L.get("mlp")
+        if mlp:
+            fk = mlp.get("kind", "dense")
+            if fk == "dense":
+                ff = dict(ff=int(mlp["ff"]), ff_kind="gated_silu")
+            elif fk == "moe":
+                r, gr = mlp["router"], mlp["router"].get("groups") or {}
+                ff = dict(ff=int(mlp["expert"]["ff"]), ff_kind="moe", router="group_score",
+                          expert_act="clamp_swish", experts=int(r["experts"]), top=int(r["top"]),
+                          router_groups=int(gr.get("count") or 1),
+                          router_keep=int(gr.get("keep") or gr.get("count") or 1),
+                          router_scale=float(r.get("scale", 1.0)),
+                          act_limit=float(mlp["expert"]["limit"]))
+                E, ng, keep = ff["experts"], ff["router_groups"], ff["router_keep"]
+                if E % ng or not 1 <= keep <= ng or not 1 <= ff["top"] <= keep * (E // ng):
+                    raise ValueError(f"layer {i}: router of {E} experts in {ng} groups, "
+                                     f"{keep} kept, top {ff['top']}")
+            else:
+                raise ValueError(f"unsupported feed-forward kind '{fk}'")
+        if kind == "lightning":
+            H = int(mx["heads"])
+            decays = tuple(float(a) for a in mx["decay"])
+            if len(decays) != H:
+                raise ValueError(f"layer {i}: {len(decays)} decays for {H} heads")
+            specs.append(LayerSpec("lightning", heads=H, dim=int(mx["dim"]),
+                                   vdim=int(mx.get("vdim", mx["dim"])), decays=decays, **ff))
+        elif kind == "parallel":
+            l, r = mx["left"], mx["right"]
+            Hl, d = int(l["heads"]), int(l["dim"])
+            G = int(l.get("kv_heads") or Hl)
+            if Hl % G:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+            rot = l.get("rot") or {}
+            sc = rot.get("scaling")
+            dims = int(rot.get("dims") or 0)
+            if dims % 2 or dims > d:
+                raise ValueError(f"layer {i}: rot.dims {dims} of a head of {d}")
+            left = LayerSpec(
+                "sink_attention", heads=Hl, kv_heads=G, dim=d, vdim=int(l.get("vdim", d)),
+                scale=float(l.get("scale", d ** -0.5)), rot_dims=dims,
+                rot_base=float(rot.get("base", 10000.0)), window=1 << 30,
+                rot_scaling=((float(sc["factor"]), float(sc["original"]), float(sc["fast"]),
+                              float(sc["slow"])) if sc else ()))
+            right = LayerSpec("mlstm", heads=int(r["heads"]), dim=int(r["dim"]),
+                              vdim=int(r.get("vdim", r["dim"])), gate_cap=float(r["gate_cap"]))
+            specs.append(LayerSpec("parallel", heads=max(Hl, right.heads), kv_heads=G,
+                                   dim=max(d, right.dim), vdim=max(left.vdim, right.vdim),
+                                   left=left, right=right,
+                                   left_scale=float(mx.get("left_scale", 1.0)),
+                                   right_scale=float(mx.get("right_scale", 1.0)), **ff))
+        else:
+            raise ValueError(f"unsupported mixer type '{kind}'")
+    lp = c.get("loop")
+    loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"])) if lp else ()
+    if loop and not (0 <= loop[0] < loop[1] <= len(specs) and loop[2] >= 1):
+        raise ValueError(f"bad loop {loop} for {len(specs)} layers")
+    return hybrid_config(name or c.get("_name_or_path") or "lapunex", int(c["width"]),
+                         int(c["vocab"]), specs, loop,
+                         norm_eps=float((c.get("norm") or {}).get("eps", 1e-5)), arch="lapunex",
+                         embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
+                         streams=int(c.get("streams") or 0), norm_offset=1.0, loop_entry=False)
+
+
 def config_from_hf(c: dict, name: Optional[str] = None) -> ModelConfig:
     """Map a ``config.json``: HF llama / mistral / mixtral / gpt2 model types, or one of the
-    native layer-list designs (``architecture``: Buborax, Pulunex, Risutar)."""
+    native layer-list designs (``architecture``: Buborax, Pulunex, Risutar, Lapunex)."""
     if c.get("architecture") == "Buborax":
         return buborax_config(c, name)
     if c.get("architecture") == "Pulunex":
         return pulunex_config(c, name)
     if c.get("architecture") == "Risutar":
         return risutar_config(c, name)
+    if c.get("architecture") == "Lapunex":
+        return lapunex_config(c, name)
     mt = c.get("model_type", "")
     name = name or c.get("_name_or_path") or mt
     if mt == "gpt2":
@@ -345,6 +424,8 @@ def load_hf_dir(d, device="cpu", dtype=torch.bfloat16, name: Optional[str] = Non
             params = from_pulunex_state_dict(cfg, sd, dtype=dtype)
         elif cfg.arch == "risutar":
             cfg, params = from_risutar_state_dict(cfg, sd, dtype=dtype)
+        elif cfg.arch == "lapunex":
+            params = from_lapunex_state_dict(cfg, sd, dtype=dtype)
         elif cfg.is_hybrid:
             params = from_buborax_state_dict(cfg, sd, dtype=dtype)
         else:

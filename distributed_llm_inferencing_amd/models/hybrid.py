@@ -1,8 +1,10 @@
-"""Hybrid decoder (archs ``buborax``, ``pulunex``, ``risutar``): a layer list that mixes
-windowed attention, latent attention, gated linear recurrences (HGRN2, gated linear attention)
-and block attention with head-mixed scores; dense, gated and routed feed-forwards; a
-shared-weight loop, grouped RMS norms, token shift and an fp32 residual stream — served by the
-same engine, scheduler, block manager and runner as the transformer families.
+"""Hybrid decoder (archs ``buborax``, ``pulunex``, ``risutar``, ``lapunex``): a layer list that
+mixes windowed attention, latent attention, gated linear recurrences (HGRN2, gated linear
+attention, fixed-decay linear attention, a matrix memory beside a sink attention) and block
+attention with head-mixed scores; dense, gated and routed feed-forwards; a shared-weight loop,
+grouped RMS norms, token shift and an fp32 residual stream (or several hyper-connected
+streams) — served by the same engine, scheduler, block manager and runner as the transformer
+families.
 
     embed (fp32) -> per layer run: x += m * mixer(gnorm(x)); x += m * ff(gnorm(x))
                  -> gnorm -> LM head (fp32 logits) -> sampler
@@ -15,6 +17,15 @@ Post-norm designs (``cfg.post_norm``; ``risutar``) run
 
 with layer norms that carry weight and bias, the sublayers reading x itself (its rounding to
 the storage dtype feeds the GEMMs; the stream, the norms and the sums stay fp32).
+
+Hyper-connected designs (``cfg.streams``; ``lapunex``) keep S copies x_1 .. x_S of the stream,
+all equal to the embedding output at first. A sublayer with read weights a, write weights b
+and stream mix M runs
+
+    u = sum_s a_s x_s;   y = sublayer(norm(u));   x_t <- sum_s M[s, t] x_s + b_t y   (all t at once)
+
+and the final norm reads the sum of the streams (``ops.hybrid.hyper_mix`` fuses a sublayer's
+write-back with the next sublayer's read and norm).
 
 * Layers [start, stop) of the loop run ``times`` times with the same weights; a pass starts
   with x = W_in [x ; x0] + step[pass] (x0 = the embedding output). Every run owns its cache or
@@ -58,6 +69,7 @@ class HybridLM(TransformerLM):
             derive_constants(spec, lp, self.device)
         self._cu: Dict[int, torch.Tensor] = {}
         self._rows: Dict[int, torch.Tensor] = {}
+        self._sum_streams: Optional[torch.Tensor] = None
         # debugging aid: when a list, forward_layers appends the residual after every run
         self.layer_trace: Optional[List[torch.Tensor]] = None
 
@@ -132,14 +144,38 @@ class HybridLM(TransformerLM):
                 self.layer_trace.append(x.clone())
         return x
 
+    def _hyper_layers(self, x: torch.Tensor, b: DeviceBatch, kv_caches) -> torch.Tensor:
+        """Pre-norm layers over hyper-connected streams; returns the sum of the streams."""
+        cfg = self.cfg
+        eps, off, S = cfg.norm_eps, cfg.norm_offset, cfg.streams
+        step = self._step_view(b, kv_caches.block_size)
+        T, D = x.shape
+        xs = x.unsqueeze(1).expand(T, S, D).contiguous()
+        if self._sum_streams is None or self._sum_streams.device != x.device:
+            self._sum_streams = torch.ones(S, dtype=torch.float32, device=x.device)
+        y = prev = None                     # a sublayer's output awaiting its write-back
+        for ri, (li, _, _) in enumerate(self.runs):
+            spec, lp = cfg.layer_specs[li], self.layers[li]
+            h = H.hyper_mix(xs, y, prev, lp["hc1"], lp["norm1"], eps, off)
+            y, prev = MIXERS[spec.kind](spec, lp, h, step, kv_caches.entries[ri], eps), lp["hc1"]
+            if spec.ff:
+                h = H.hyper_mix(xs, y, prev, lp["hc2"], lp["norm2"], eps, off)
+                y, prev = FEED_FORWARDS[spec.ff_kind](spec, lp, h), lp["hc2"]
+            if self.layer_trace is not None:
+                self.layer_trace.append(H.hyper_mix(xs, y, prev, self._sum_streams, None))
+                y = prev = None
+        return H.hyper_mix(xs, y, prev, self._sum_streams, None)
+
     def forward_layers(self, x: torch.Tensor, b: DeviceBatch, kv_caches) -> torch.Tensor:
         cfg, p = self.cfg, self.params
         if cfg.post_norm:
             return self._postnorm_layers(x, b, kv_caches)
-        eps, groups, m = cfg.norm_eps, cfg.norm_groups, cfg.residual_mult
+        if cfg.streams:
+            return self._hyper_layers(x, b, kv_caches)
+        eps, groups, m, off = cfg.norm_eps, cfg.norm_groups, cfg.residual_mult, cfg.norm_offset
         step = self._step_view(b, kv_caches.block_size)
         entries = kv_caches.entries
-        x0 = x.clone() if cfg.loop else None
+        x0 = x.clone() if cfg.loop and cfg.loop_entry else None
         pending = None                      # a sub-block's fp32 output awaiting its add
         for ri, (li, t, first) in enumerate(self.runs):
             spec, lp = cfg.layer_specs[li], self.layers[li]
@@ -152,13 +188,13 @@ class HybridLM(TransformerLM):
                                        bias=p["loop_step"][t], out_f32=spec.shift)
             else:
                 h = H.resadd_groupnorm(x, pending, lp["norm1"], groups, eps, mult=m,
-                                       out_f32=spec.shift)
+                                       out_f32=spec.shift, w_offset=off)
             if spec.shift:                  # the mixer reads the rows mixed with their predecessors
                 h = H.token_shift(h, lp["shift"], kv_caches.shift_states[ri], step.state_slots,
                                   step.cu_seqlens, step.max_seqlen, step.positions)
             y = MIXERS[spec.kind](spec, lp, h, step, entries[ri], eps)
             if spec.ff:
-                h = H.resadd_groupnorm(x, y, lp["norm2"], groups, eps, mult=m)
+                h = H.resadd_groupnorm(x, y, lp["norm2"], groups, eps, mult=m, w_offset=off)
                 y = FEED_FORWARDS[spec.ff_kind](spec, lp, h)
             pending = y
             if self.layer_trace is not None:
@@ -184,10 +220,11 @@ class HybridLM(TransformerLM):
                               rows_idx=rows)
         if rows is None:
             return H.resadd_groupnorm(hidden, None, p["final_norm"], cfg.norm_groups,
-                                      cfg.norm_eps, gain=cfg.logit_scale)
+                                      cfg.norm_eps, gain=cfg.logit_scale,
+                                      w_offset=cfg.norm_offset)
         # the logit scale rides on the final norm's output: the head is linear
         return H.groupnorm_rows(hidden, rows, p["final_norm"], cfg.norm_groups, cfg.norm_eps,
-                                gain=cfg.logit_scale)
+                                gain=cfg.logit_scale, w_offset=cfg.norm_offset)
 
     def head_logits(self, h: torch.Tensor) -> torch.Tensor:
         return H.linear_any(h, self.params["lm_head"], out_f32=True)

@@ -48,10 +48,39 @@ def derive_constants(spec: LayerSpec, lp: dict, device) -> None:
         lp["inv_freq"] = torch.pow(spec.rot_base, -2.0 * i / max(1, spec.rot_dims)).to(device)
     elif spec.kind == "talk_attention":
         lp["talk"] = lp["talk"].float().contiguous()
-    if spec.ff_kind == "moe" and spec.ff and spec.router == "score":
+    elif spec.kind == "lightning":
+        lp["decays"] = torch.tensor(spec.decays, dtype=torch.float64).float().to(device)
+    elif spec.kind == "parallel":
+        freq, mscale = yarn_frequencies(spec.left.rot_dims, spec.left.rot_base,
+                                        spec.left.rot_scaling)
+        lp["rot_freq"], lp["rot_mscale"] = freq.to(device), mscale
+        lp["sink"] = lp["sink"].float().contiguous()
+        lp["if_b"] = lp["if_b"].float().contiguous()
+    if spec.ff_kind == "moe" and spec.ff and spec.router == "score" and "correction" in lp:
         lp["correction"] = lp["correction"].float().contiguous()
     if spec.ff_kind == "moe" and spec.ff and spec.router == "logit_topk":
         lp["router_b"] = lp["router_b"].float().contiguous()
+
+
+def yarn_frequencies(dims: int, base: float, scaling: tuple = ()):
+    """(float64 frequency of every rotated pair, factor on cos and sin). Pair i turns by
+    position * base^(-2i/dims). With YaRN scaling (factor, original length, fast turns, slow
+    turns) a pair that makes more than ``fast`` turns over the original length keeps its
+    frequency, one that makes fewer than ``slow`` is slowed by ``factor``, with a linear ramp
+    over the pair index between the two, and cos / sin grow by 0.1 ln(factor) + 1."""
+    import math
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(base, dtype=torch.float64), -2.0 * i / max(1, dims))
+    if not scaling or not dims:
+        return f, 1.0
+    factor, orig, fast, slow = scaling
+
+    def pair_at(turns):          # the (fractional) pair index that makes this many turns
+        return dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+    lo = max(math.floor(pair_at(fast)), 0)
+    hi = min(math.ceil(pair_at(slow)), dims - 1)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return f / factor * ramp + f * (1.0 - ramp), 0.1 * math.log(factor) + 1.0
 
 
 def attention_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, eps: float):
@@ -157,9 +186,49 @@ def talk_attention_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, ep
     return H.linear_any(o, lp["wo"])
 
 
+def lightning_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, eps: float):
+    """Linear attention with one fixed decay per head: SiLU on q / k / v, the state and its
+    read-out in fp32, all heads RMS-normed together, sigmoid output gate."""
+    (state,) = cache
+    Hh, d, dv = spec.heads, spec.dim, spec.vdim
+    proj = H.linear_any(h, lp["w_in"])                       # fp32 [T, q | k | v | gate]
+    o = H.lightning(proj, lp["decays"], state, step.state_slots, step.cu_seqlens,
+                    step.max_seqlen, step.positions, Hh, d, dv)
+    g0 = 2 * Hh * d + Hh * dv
+    return H.linear_any(H.rmsnorm_cols(o, lp["o_norm"], eps, gate=proj[:, g0:g0 + Hh * dv]),
+                        lp["wo"])
+
+
+def parallel_mixer(spec: LayerSpec, lp: dict, h, step: StepView, cache, eps: float):
+    """Two mixers on the same input, summed with fixed scales: causal grouped-query attention
+    (whole-row q / k norm, partial rotation, a sink logit per head, a sigmoid gate per head)
+    and a matrix memory with exponential gating. One fused input projection; both sides write
+    their gated, scaled outputs side by side, so one output GEMM over [left | right] sums them."""
+    l, r = spec.left, spec.right
+    kc, vc, state, mstate = cache
+    T = h.shape[0]
+    proj = H.linear_any(h, lp["w_in"])
+    nl = l.heads * l.dim + l.kv_heads * (l.dim + l.vdim)
+    q = H.sink_prepare(proj, lp["q_norm"], lp["k_norm"], eps, l.heads, l.kv_heads, l.dim,
+                       l.vdim, l.rot_dims, lp["rot_freq"], lp["rot_mscale"], step.positions,
+                       kc, vc, step.slot_mapping)
+    wl, wr = l.heads * l.vdim, r.heads * r.vdim
+    o = torch.empty(T, wl + wr, dtype=h.dtype, device=h.device)
+    # causal, unwindowed: a window as long as the step's longest context masks nothing
+    win = min(l.window or (1 << 30), max(1, step.max_context))
+    H.window_attention(q, kc, vc, l.dim, l.vdim, l.heads, l.kv_heads, step.cu_seqlens,
+                       step.max_seqlen, step.positions, step.block_tables, step.block_size,
+                       win, l.scale, gate=proj[:, nl:nl + l.heads], sink=lp["sink"],
+                       head_gate=True, out_scale=spec.left_scale, out=o[:, :wl])
+    H.mlstm(proj[:, nl + l.heads:], lp["if_b"], r.gate_cap, lp["o_norm"], eps, state, mstate,
+            step.state_slots, step.cu_seqlens, step.max_seqlen, step.positions, r.heads, r.dim,
+            r.vdim, o[:, wl:], spec.right_scale)
+    return H.linear_any(o, lp["wo"])
+
+
 MIXERS = {"attention": attention_mixer, "hgrn2": hgrn2_mixer,
           "latent_attention": latent_attention_mixer, "talk_attention": talk_attention_mixer,
-          "gla": gla_mixer}
+          "gla": gla_mixer, "lightning": lightning_mixer, "parallel": parallel_mixer}
 
 
 # ----------------------------------------------------------------------------- feed-forwards
@@ -178,6 +247,7 @@ def prepare_feed_forward(spec: LayerSpec, params: dict, pre: str) -> None:
     w = params.get(pre + "w_down")
     if (not spec.ff or w is None or pre + "ff_tuned" in params or w.dtype != torch.bfloat16
             or not w.is_cuda or spec.ff_kind not in ("gelu", "moe", "gated_silu")
+            or spec.expert_act == "clamp_swish"
             or w.shape[-2] % 64 or spec.ff % 64 or spec.shared_ff % 64):
         return
     if spec.ff_kind == "gelu":
@@ -221,7 +291,13 @@ def gated_silu_ff(spec: LayerSpec, lp: dict, h):
 def moe_ff(spec: LayerSpec, lp: dict, h):
     """Routed gated-SiLU experts + identity experts + a gated shared expert, summed in fp32;
     with ``router`` = ``logit_topk``: biased logits, softmax over the chosen, ungated exact-GELU
-    experts and an always-on shared expert."""
+    experts and an always-on shared expert; with ``router`` = ``group_score``: group-limited
+    choice, scaled scores, clamped-swish experts."""
+    if spec.router == "group_score":
+        tw, ti, _ = H.score_router(h, lp["router"], None, spec.top, 0, spec.router_groups,
+                                   spec.router_keep, spec.router_scale)
+        return H.moe_experts_f32(h, lp["w_gu"], lp["w_down"], tw, ti, None, act="clamp_swish",
+                                 limit=spec.act_limit)
     if spec.router == "logit_topk":
         tw, ti = H.logit_router(h, lp["router"], lp["router_b"], spec.top)
         if "ff_tuned" not in lp:

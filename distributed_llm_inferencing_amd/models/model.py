@@ -62,7 +62,8 @@ class TransformerLM:
         le = cfg.num_layers if layer_end is None else layer_end
         shapes = W.stage_param_shapes(cfg, layer_start, le, layer_start == 0,
                                       le == cfg.num_layers, None)
-        params = W.random_init(shapes, device, dtype, seed)
+        params = W.random_init(shapes, device, dtype, seed,
+                                norm_value=1.0 - cfg.norm_offset)
         if expert_range is not None:
             params = {k: W.slice_experts(k, v, expert_range) for k, v in params.items()}
         return cls(cfg, params, layer_start, le, device, expert_range)

@@ -54,8 +54,20 @@ def hybrid_layer_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
       latent_attention with ``q_rank`` / ``head_gate``: w_in [rq + (r + dr) + H, D] = query
                         latent | compressed kv (absent with ``kv_from``) | head gates,
                         q_norm [rq], w_uq [H*(d+dr), rq], then as above
+      lightning:        w_in [2*H*d + 2*H*dv, D] = q | k | v | output gate, o_norm [H*dv],
+                        wo [D, H*dv]
+      parallel:         w_in = left q [Hl*d] | left k [G*d] | left v [G*dvl] | left head gates
+                        [Hl] | right q [Hr*dr] | right k [Hr*dr] | right v [Hr*dvr] | right
+                        output gate [Hr*dvr] | right input gates [Hr] | right forget gates [Hr],
+                        q_norm [Hl*d], k_norm [G*d], sink [Hl] fp32, o_norm [Hr*dvr],
+                        if_b [2*Hr] fp32 (input | forget gate biases),
+                        wo [D, Hl*dvl + Hr*dvr] = left | right output projections
+        moe, router ``group_score`` with ``clamp_swish`` experts: router [E, D],
+                        w_gu [E, 2F, D], w_down [E, D, F]
     Post-norm designs add the norms' biases norm1_b / norm2_b [D]; with a per-layer token input
-    of width s: side_gate [s, D], side_proj [D, s], side_norm [D]."""
+    of width s: side_gate [s, D], side_proj [D, s], side_norm [D]. With hyper-connections over
+    S streams every sublayer has hc1 / hc2 fp32 [S + S + S*S] = read weights | write weights |
+    stream mix [from, to]."""
     D = cfg.hidden_size
     s = cfg.layer_specs[i]
     p = f"layers.{i}."
@@ -85,8 +97,24 @@ def hybrid_layer_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
         n_in = H * d + (0 if s.kv_from >= 0 else s.kv_heads * (d + dv))
         out.update({p + "shift": (D,), p + "w_in": (n_in, D), p + "b_in": (n_in,),
                     p + "talk": (H, H), p + "wo": (D, H * dv)})
+    elif s.kind == "lightning":
+        out.update({p + "w_in": (2 * H * (d + dv), D), p + "o_norm": (H * dv,),
+                    p + "wo": (D, H * dv)})
+    elif s.kind == "parallel":
+        l, r = s.left, s.right
+        n_in = (l.heads * l.dim + l.kv_heads * (l.dim + l.vdim) + l.heads
+                + r.heads * (2 * r.dim + 2 * r.vdim + 2))
+        out.update({p + "w_in": (n_in, D), p + "q_norm": (l.heads * l.dim,),
+                    p + "k_norm": (l.kv_heads * l.dim,), p + "sink": (l.heads,),
+                    p + "o_norm": (r.heads * r.vdim,), p + "if_b": (2 * r.heads,),
+                    p + "wo": (D, l.heads * l.vdim + r.heads * r.vdim)})
     else:
         raise ValueError(f"unknown mixer kind '{s.kind}'")
+    if cfg.streams:
+        n = cfg.streams * (cfg.streams + 2)
+        out[p + "hc1"] = (n,)
+        if s.ff:
+            out[p + "hc2"] = (n,)
     if cfg.post_norm:
         out[p + "norm1_b"] = (D,)
         if s.ff:
@@ -103,6 +131,9 @@ def hybrid_layer_shapes(cfg: ModelConfig, i: int) -> Dict[str, tuple]:
         out.update({p + "norm2": (D,), p + "w_gu": (2 * s.ff, D), p + "w_down": (D, s.ff)})
     elif s.ff and s.ff_kind == "gelu":
         out.update({p + "norm2": (D,), p + "w_up": (s.ff, D), p + "w_down": (D, s.ff)})
+    elif s.ff and s.ff_kind == "moe" and s.router == "group_score":
+        out.update({p + "norm2": (D,), p + "router": (s.experts, D),
+                    p + "w_gu": (s.experts, 2 * s.ff, D), p + "w_down": (s.experts, D, s.ff)})
     elif s.ff and s.ff_kind == "moe":
         n = s.experts + s.identity
         out.update({p + "norm2": (D,), p + "router": (n + (1 if s.shared_ff else 0), D),
@@ -141,7 +172,7 @@ def global_param_shapes(cfg: ModelConfig, first: bool, last: bool) -> Dict[str, 
         # the loop entry re-reads the embedding output, so a stage that runs loop layers
         # holds the embedding too (hybrid designs run on one stage)
         s.update({"embed": (v, d), "final_norm": (d,), "lm_head": (v, d)})
-        if cfg.loop:
+        if cfg.loop and cfg.loop_entry:
             s.update({"loop_in": (d, 2 * d), "loop_step": (cfg.loop[2], d)})
         if cfg.learned_pos:
             s["pos_embed"] = (cfg.max_position, d)
@@ -190,7 +221,7 @@ def _is_bias(name: str) -> bool:
 
 
 def random_init(shapes: Dict[str, tuple], device, dtype=torch.bfloat16, seed: int = 0,
-                std: float = INIT_STD) -> Dict[str, torch.Tensor]:
+                std: float = INIT_STD, norm_value: float = 1.0) -> Dict[str, torch.Tensor]:
     """Deterministic per-tensor init: each tensor's values depend only on (seed, name), so a
     pipeline stage generates exactly the slice the full model would hold."""
     out = {}
@@ -201,7 +232,9 @@ def random_init(shapes: Dict[str, tuple], device, dtype=torch.bfloat16, seed: in
         if hybrid and not _is_norm_weight(name) and not _is_bias(name):
             out[name] = _hybrid_init(name, shape, dev, dtype, seed)
         elif _is_norm_weight(name):
-            out[name] = torch.ones(shape, dtype=dtype, device=dev)
+            # a design that stores its layer norms' weights as offsets starts them at zero
+            v = norm_value if name.endswith(("norm1", "norm2", "final_norm")) else 1.0
+            out[name] = torch.full(shape, v, dtype=dtype, device=dev)
         elif _is_bias(name):
             out[name] = torch.zeros(shape, dtype=dtype, device=dev)
         else:
@@ -227,6 +260,21 @@ def _hybrid_init(name: str, shape: tuple, dev, dtype, seed: int) -> torch.Tensor
         return (0.05 * torch.randn(shape, generator=g)).to(dev, torch.float32)
     if name.endswith(".router_b"):
         return (0.1 * torch.randn(shape, generator=g)).to(dev, torch.float32)
+    if name.endswith((".hc1", ".hc2")):
+        # read weights near 1/S, write weights near 1, a stream mix near the identity
+        S = int(round((1 + shape[0]) ** 0.5)) - 1
+        t = torch.cat([torch.full((S,), 1.0 / S) + 0.1 * torch.randn(S, generator=g),
+                       1.0 + 0.2 * torch.randn(S, generator=g),
+                       (torch.eye(S) + 0.15 * torch.randn(S, S, generator=g)).reshape(-1)])
+        return t.to(dev, torch.float32)
+    if name.endswith(".sink"):
+        return torch.randn(shape, generator=g).to(dev, torch.float32)
+    if name.endswith(".if_b"):
+        # input gates around -1, forget gates around +3 (slow forgetting)
+        H = shape[0] // 2
+        t = torch.cat([-1.0 + 0.5 * torch.randn(H, generator=g),
+                       3.0 + 1.0 * torch.randn(H, generator=g)])
+        return t.to(dev, torch.float32)
     if name.endswith(".a_b"):
         # decays sigmoid(z)^(1/tau) spread between fast and slow channels
         return (1.0 + 2.0 * torch.randn(shape, generator=g)).to(dev, dtype)
@@ -485,3 +533,61 @@ def from_risutar_state_dict(cfg: ModelConfig, sd, dtype=torch.bfloat16):
         if s.shared_ff:
             out[p + "ws_up"], out[p + "ws_down"] = cv(sd[f + "shared.up"]), cv(sd[f + "shared.down"])
     return replace(cfg, layer_specs=tuple(specs)), out
+
+
+# ----------------------------------------------------------------------------- Lapunex files
+def from_lapunex_state_dict(cfg: ModelConfig, sd, dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Convert a Lapunex checkpoint (tensor names ``embed``, ``head``, ``final.norm``,
+    ``l<i>.norm1|norm2``, ``l<i>.hc1|hc2.in|out|mix``, ``l<i>.mix.*`` (``left.*`` / ``right.*``
+    in a parallel layer), ``l<i>.mlp.gate|up|down`` or ``l<i>.mlp.router|e<j>.gate|up|down``;
+    linear weights [out, in]) into the layout of ``hybrid_layer_shapes``: all projections that
+    read the mixer's input are stacked into one matrix, the two output projections of a
+    parallel layer side by side into another, the experts are stacked, and a sublayer's
+    hyper-connection tensors become one fp32 vector. Norm weights stay as stored (offsets from
+    one; the kernels add the one in fp32)."""
+    cv = lambda t: t.detach().to(dtype).contiguous()  # noqa: E731
+    f32 = lambda t: t.detach().float().reshape(-1)  # noqa: E731
+    out = {"embed": cv(sd["embed"]), "lm_head": cv(sd["head"]), "final_norm": cv(sd["final.norm"])}
+    for i, s in enumerate(cfg.layer_specs):
+        a, p = f"l{i}.", f"layers.{i}."
+        m = a + "mix."
+        out[p + "norm1"] = cv(sd[a + "norm1"])
+        for q in ("1", "2") if cfg.streams else ():
+            if q == "2" and not s.ff:
+                continue
+            h = f"{a}hc{q}."
+            if tuple(sd[h + "mix"].shape) != (cfg.streams, cfg.streams):
+                raise ValueError(f"{h}mix: not [{cfg.streams}, {cfg.streams}]")
+            out[p + "hc" + q] = torch.cat([f32(sd[h + "in"]), f32(sd[h + "out"]),
+                                           f32(sd[h + "mix"])]).contiguous()
+        if s.kind == "lightning":
+            out[p + "w_in"] = cv(torch.cat([sd[m + n] for n in "qkvg"], 0))
+            out[p + "o_norm"] = cv(sd[m + "norm"])
+            out[p + "wo"] = cv(sd[m + "o"])
+        else:
+            lt, rt = m + "left.", m + "right."
+            out[p + "w_in"] = cv(torch.cat([sd[lt + n] for n in "qkvg"]
+                                           + [sd[rt + n] for n in "qkvgif"], 0))
+            out[p + "q_norm"], out[p + "k_norm"] = cv(sd[lt + "q.norm"]), cv(sd[lt + "k.norm"])
+            out[p + "sink"] = f32(sd[lt + "sink"]).contiguous()
+            out[p + "o_norm"] = cv(sd[rt + "norm"])
+            out[p + "if_b"] = torch.cat([f32(sd[rt + "i.b"]), f32(sd[rt + "f.b"])]).contiguous()
+            out[p + "wo"] = cv(torch.cat([sd[lt + "o"], sd[rt + "o"]], 1))
+        if not s.ff:
+            continue
+        f = a + "mlp."
+        out[p + "norm2"] = cv(sd[a + "norm2"])
+        if s.ff_kind == "gated_silu":
+            out[p + "w_gu"] = cv(torch.cat([sd[f + "gate"], sd[f + "up"]], 0))
+            out[p + "w_down"] = cv(sd[f + "down"])
+            continue
+        out[p + "router"] = cv(sd[f + "router"])
+        out[p + "w_gu"] = cv(torch.stack([torch.cat([sd[f"{f}e{e}.gate"], sd[f"{f}e{e}.up"]], 0)
+                                          for e in range(s.experts)]))
+        out[p + "w_down"] = cv(torch.stack([sd[f"{f}e{e}.down"] for e in range(s.experts)]))
+    want = stage_param_shapes(cfg, 0, len(cfg.layer_specs), True, True)
+    for k, shp in want.items():
+        if k not in out or tuple(out[k].shape) != tuple(shp):
+            got = tuple(out[k].shape) if k in out else None
+            raise ValueError(f"{k}: the checkpoint gives {got}, the configuration {tuple(shp)}")
+    return out

@@ -74,20 +74,20 @@ _SIGS = {
     # hybrid family (ops/hybrid.py)
     "dli_gemm_any": [P, L, P, L, P, L, I, I, I, I, I, I, L, L, L, P],
     "dli_embedding_f32": [P, P, P, P, I, I, I, F, P, P, I, I, P],
-    "dli_resadd_groupnorm": [P, P, I, P, F, F, P, P, I, I, I, I, F, P, F, I, I, P],
+    "dli_resadd_groupnorm": [P, P, I, P, F, F, P, P, I, I, I, I, F, P, F, I, F, I, P],
     "dli_token_shift": [P, P, P, P, P, P, P, I, I, I, I, P],
-    "dli_act_mul": [P, I, P, I, I, I, I, P, I, P],
+    "dli_act_mul": [P, I, P, I, I, I, I, P, F, I, P],
     "dli_talk_prepare": [P, I, P, P, F, I, I, I, I, I, P, P, P, P, I, P],
-    "dli_score_router": [P, P, P, P, I, P, P, I, I, I, I, I, I, P],
+    "dli_score_router": [P, P, P, P, I, P, P, I, I, I, I, I, I, I, F, I, P],
     "dli_gemm_any_grouped": [P, L, P, L, L, P, L, I, I, I, I, I, P, P, P],
     "dli_moe_combine_f32": [P, P, P, P, P, P, P, I, P, P, I, I, I, I, I, I, P],
     "dli_concat_cast": [P, P, P, I, I, I, P],
     "dli_attn_prepare": [P, I, P, P, F, I, I, I, I, P, P, P, P, I, P],
     "dli_mla_prepare": [P, I, P, F, I, I, I, I, I, I, P, P, P, P, P, P, I, P],
     "dli_window_attention": [P, I, P, L, P, L, P, I, P, I, P, P, P, P, P,
-                             I, I, I, I, I, I, I, I, I, F, I, I, I, P],
+                             I, I, I, I, I, I, I, I, I, F, I, I, P, I, F, I, P],
     "dli_window_attention_mfma": [P, I, P, L, P, L, P, I, P, I, P, P, P, P, P,
-                                  I, I, I, I, I, I, I, I, I, F, I, P, I, I, I, P],
+                                  I, I, I, I, I, I, I, I, I, F, I, P, I, I, I, P, I, F, P],
     "dli_window_attention_mfma_workspace_bytes": [I, I, I, I, I, I, I, I],
     "dli_hgrn2": [P, I, P, P, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P],
     "dli_gla": [P, I, P, I, P, F, F, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P],
@@ -97,10 +97,15 @@ _SIGS = {
     "dli_postnorm": [P, P, I, F, P, P, P, I, I, F, P, I, P],
     "dli_add_rmsnormed": [P, P, I, P, P, I, I, F, I, P],
     "dli_side_gate": [P, P, I, P, P, I, I, I, I, I, I, P],
-    "dli_rmsnorm_cols": [P, P, I, P, I, I, F, I, P],
+    "dli_rmsnorm_cols": [P, P, I, P, I, I, F, P, I, I, P],
     "dli_latent_prepare": [P, I, P, I, P, F, I, I, I, I, I, I, P, P, P, P, P, P, I, I, P],
     "dli_head_gate": [P, P, P, I, I, I, I, I, P],
     "dli_logit_router": [P, P, P, I, P, P, I, I, I, I, I, P],
+    # hyper-connected designs (streams.hip, recurrent_scalar.hip)
+    "dli_hyper_mix": [P, P, I, P, P, P, P, I, I, I, F, F, I, P],
+    "dli_sink_prepare": [P, I, P, P, F, I, I, I, I, I, I, P, F, P, P, P, P, P, I, P],
+    "dli_scalar_recurrence": [P, I, I, P, P, F, P, F, P, P, P, P, P, P, I, F, I, I, I, I, I,
+                              I, P],
 }
 
 

@@ -108,10 +108,11 @@ def embedding_f32(ids: torch.Tensor, table: torch.Tensor, copy: bool = False,
 def resadd_groupnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: Optional[torch.Tensor],
                      groups: int, eps: float, mult: float = 1.0, keep: float = 1.0,
                      bias: Optional[torch.Tensor] = None, dtype=None, gain: float = 1.0,
-                     out_f32: bool = False) -> Optional[torch.Tensor]:
+                     out_f32: bool = False, w_offset: float = 0.0) -> Optional[torch.Tensor]:
     """In place on the fp32 stream: x = keep * x + mult * y + bias (y, bias optional); returns
     the grouped RMS norm of the new x times ``w`` times ``gain`` in the storage dtype (None when
-    w is None), or unrounded in fp32 with ``out_f32`` (what a token shift reads)."""
+    w is None), or unrounded in fp32 with ``out_f32`` (what a token shift reads). ``w_offset``
+    is added to the weight in fp32 (weights stored as offsets from one)."""
     dtype = dtype or (w.dtype if w is not None else torch.bfloat16)
     if not x.is_cuda:
         if keep != 1.0:
@@ -122,7 +123,7 @@ def resadd_groupnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: Optional[tor
             x.add_(bias.float())
         if w is None:
             return None
-        h = R.group_rmsnorm(x, w, groups, eps, torch.float32)
+        h = R.group_rmsnorm(x, w, groups, eps, torch.float32, w_offset)
         if gain != 1.0:
             h = h * gain
         return h if out_f32 else h.to(dtype)
@@ -131,20 +132,20 @@ def resadd_groupnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: Optional[tor
          if w is not None else None)
     _call("dli_resadd_groupnorm", _p(x), _p(y), y.stride(0) if y is not None else 0, _p(bias),
           float(keep), float(mult), _p(w), _p(h), dim, rows, dim, groups, float(eps), None,
-          float(gain), int(out_f32), _dt(dtype), _st())
+          float(gain), int(out_f32), float(w_offset), _dt(dtype), _st())
     return h
 
 
 def groupnorm_rows(x: torch.Tensor, rows_idx: torch.Tensor, w: torch.Tensor, groups: int,
-                   eps: float, gain: float = 1.0) -> torch.Tensor:
+                   eps: float, gain: float = 1.0, w_offset: float = 0.0) -> torch.Tensor:
     """Grouped RMS norm (times ``gain``) of the rows ``rows_idx`` (int64) of the fp32 stream."""
     if not x.is_cuda:
-        h = R.group_rmsnorm(x.index_select(0, rows_idx), w, groups, eps, torch.float32)
+        h = R.group_rmsnorm(x.index_select(0, rows_idx), w, groups, eps, torch.float32, w_offset)
         return (h * gain if gain != 1.0 else h).to(w.dtype)
     n, dim = rows_idx.shape[0], x.shape[1]
     h = torch.empty(n, dim, dtype=w.dtype, device=x.device)
     _call("dli_resadd_groupnorm", _p(x), None, 0, None, 1.0, 1.0, _p(w), _p(h), dim, n, dim,
-          groups, float(eps), _p(rows_idx), float(gain), 0, _dt(w.dtype), _st())
+          groups, float(eps), _p(rows_idx), float(gain), 0, float(w_offset), _dt(w.dtype), _st())
     return h
 
 
@@ -174,21 +175,24 @@ def concat_cast(a: torch.Tensor, b: torch.Tensor, dtype) -> torch.Tensor:
     return out
 
 
-_ACT_KINDS = {"gelu_mul": 0, "silu_mul": 1, "gelu": 2, "gelu_erf": 3, "copy": 4}
+_ACT_KINDS = {"gelu_mul": 0, "silu_mul": 1, "gelu": 2, "gelu_erf": 3, "copy": 4,
+              "clamp_swish": 5}
 
 
 def act_mul(gu: torch.Tensor, F_: int, dtype, kind: str = "gelu_mul",
-            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+            rows: Optional[torch.Tensor] = None, limit: float = 0.0) -> torch.Tensor:
     """The feed-forward's middle for an fp32 projection: ``gelu_mul`` / ``silu_mul`` =
     act(gu[:, :F]) * gu[:, F:2F]; ``gelu`` = gelu_tanh(gu[:, :F]); ``gelu_erf`` = the exact GELU
-    of gu[:, :F]; ``copy`` = gu[:, :F] rounded to the storage dtype. ``rows`` (device int32
+    of gu[:, :F]; ``copy`` = gu[:, :F] rounded to the storage dtype; ``clamp_swish`` = g
+    sigmoid(1.702 g) (u + 1) with g = min(gu[:, :F], limit), u = clamp(gu[:, F:2F], +-limit).
+    ``rows`` (device int32
     scalar): only that many leading rows hold data (routed rows of a mixture)."""
     if not gu.is_cuda:
-        return R.act_mul(gu, F_, dtype, kind)
+        return R.act_mul(gu, F_, dtype, kind, limit)
     T = gu.shape[0]
     out = torch.empty(T, F_, dtype=dtype, device=gu.device)
     _call("dli_act_mul", _p(out), F_, _p(gu), gu.stride(0), T, F_, _ACT_KINDS[kind], _p(rows),
-          _dt(dtype), _st())
+          float(limit), _dt(dtype), _st())
     return out
 
 
@@ -247,27 +251,38 @@ def mla_prepare(proj, cw, eps, H, d, dr, r, rot_dims, inv_freq, positions, slots
 
 def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, positions,
                      block_tables, block_size, window, scale, slopes=None, talk=None, gate=None,
-                     chunk: int = 0, k_groups: Optional[int] = None):
+                     chunk: int = 0, k_groups: Optional[int] = None, sink=None,
+                     head_gate: bool = False, out_scale: float = 1.0, out=None):
     """See ``reference.window_attention`` / window_attention.hip. q [T, H*dq] (storage dtype);
     caches are token-major rows; returns [T, H*dv] in the storage dtype. ``chunk`` > 0 limits
     a query to the keys of its own block of that many positions; ``k_groups`` is the number of
-    key heads per cache row when it is not the number of value heads G."""
+    key heads per cache row when it is not the number of value heads G. ``sink`` fp32 [H]
+    adds exp(sink_h) to head h's softmax denominator; ``head_gate``: the gate is fp32 [T, H],
+    one number per head; ``out_scale`` multiplies the output; ``out`` (rows of a wider buffer)
+    receives it."""
     Gk = G if k_groups is None else int(k_groups)
     chunk = int(chunk)
     if not q.is_cuda:
-        return R.window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, positions,
-                                  block_tables, block_size, window, scale, slopes, talk, gate,
-                                  out_dtype=q.dtype, chunk=chunk, k_groups=Gk)
+        o = R.window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, positions,
+                               block_tables, block_size, window, scale, slopes, talk, gate,
+                               out_dtype=q.dtype, chunk=chunk, k_groups=Gk, sink=sink,
+                               head_gate=head_gate, out_scale=out_scale)
+        if out is not None:
+            out.copy_(o)
+            return out
+        return o
     T = q.shape[0]
     S = cu_seqlens.shape[0] - 1
-    out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    hg = int(bool(head_gate))
     if q.dtype == torch.bfloat16 and MFMA_ATTENTION:
         # the MFMA form; shapes it does not take (odd head sizes, > 32 heads) fall through
         lib = N.require_native()
         # decode steps of heads that share one cached row per position (latent attention):
         # the heads become the query rows of a one-head problem
         rowhead = int(Gk == 1 and H > 1 and int(max_seqlen) == 1 and talk is None and gate is None
-                      and slopes is None and q.stride(0) == H * dq)
+                      and slopes is None and sink is None and q.stride(0) == H * dq)
         nb = lib.dli_window_attention_mfma_workspace_bytes(S, int(max_seqlen), T, H, dv,
                                                            int(min(window, chunk) if chunk else window),
                                                            int(talk is not None), rowhead)
@@ -277,7 +292,7 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
             _p(out), out.stride(0), _p(gate), gate.stride(0) if gate is not None else 0,
             _p(slopes), _p(talk), _p(cu_seqlens), _p(positions), _p(block_tables),
             block_tables.stride(0), block_size, S, int(max_seqlen), H, G, dq, dv, int(window),
-            float(scale), T, _p(ws), rowhead, Gk, chunk, _st())
+            float(scale), T, _p(ws), rowhead, Gk, chunk, _p(sink), hg, float(out_scale), _st())
         if rc == 0:
             return out
         if rc != _NOT_SUPPORTED:
@@ -286,8 +301,8 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, max_seqlen, 
           _p(v_cache), v_cache.stride(0), _p(out), out.stride(0), _p(gate),
           gate.stride(0) if gate is not None else 0, _p(slopes), _p(talk), _p(cu_seqlens),
           _p(positions), _p(block_tables), block_tables.stride(0), block_size, S,
-          int(max_seqlen), H, G, dq, dv, int(window), float(scale), Gk, chunk, _dt(q.dtype),
-          _st())
+          int(max_seqlen), H, G, dq, dv, int(window), float(scale), Gk, chunk, _p(sink), hg,
+          float(out_scale), _dt(q.dtype), _st())
     return out
 
 
@@ -307,11 +322,17 @@ def hgrn2(proj, f_bias, lower, norm_w, eps, state, slots, cu_seqlens, max_seqlen
 
 
 # ----------------------------------------------------------------------------- mixture of experts
-def score_router(h, w_router, correction, top: int, n_gate: int = 0):
+def score_router(h, w_router, correction, top: int, n_gate: int = 0, groups: int = 1,
+                 keep: int = 1, wscale: float = 1.0):
     """Router with un-renormalised softmax weights and a choice correction (see
     ``reference.score_router``): (weights fp32 [T, top], ids int32 [T, top], gates fp32
-    [T, n_gate]) from one pass over each token's row, logits in fp32."""
+    [T, n_gate]) from one pass over each token's row, logits in fp32. With ``groups`` > 1 only
+    the experts of the ``keep`` best groups of neighbours can be chosen (a group scores its
+    best expert; ``reference.group_router``); ``wscale`` multiplies the weights."""
     if not h.is_cuda:
+        if groups > 1 or wscale != 1.0 or correction is None:
+            tw, ti = R.group_router(h, w_router, top, groups, keep, wscale)
+            return tw, ti, None
         return R.score_router(h, w_router, correction, top, n_gate)
     T, D = h.shape
     n = w_router.shape[0] - n_gate
@@ -319,7 +340,8 @@ def score_router(h, w_router, correction, top: int, n_gate: int = 0):
     ids = torch.empty(T, top, dtype=torch.int32, device=h.device)
     gates = torch.empty(T, max(n_gate, 1), dtype=torch.float32, device=h.device)
     _call("dli_score_router", _p(w), _p(ids), _p(gates), _p(h), h.stride(0), _p(w_router),
-          _p(correction), T, D, n, n_gate, top, _dt(h.dtype), _st())
+          _p(correction), T, D, n, n_gate, top, int(groups), int(keep), float(wscale),
+          _dt(h.dtype), _st())
     return w, ids, gates[:, :n_gate]
 
 
@@ -335,13 +357,14 @@ def grouped_linear_any(x, w, offsets, src, n: int) -> torch.Tensor:
     return out
 
 
-def moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared=None) -> torch.Tensor:
+def moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared=None, act: str = "silu_mul",
+                    limit: float = 0.0) -> torch.Tensor:
     """Weighted sum of every token's chosen experts in fp32 (``reference.moe_experts_f32``):
     ids below E run the gated-SiLU experts as grouped GEMMs over the rows sorted by expert, ids
     from E on are identity experts; ``shared`` = (ws_gu, ws_down, gate [T]) adds the always-on
     expert times its gate. No host synchronisation: a captured graph replays it."""
     if not x.is_cuda:
-        return R.moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared)
+        return R.moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared, act, limit)
     T, D = x.shape
     k = topk_ids.shape[1]
     E, F2, _ = w_gu.shape
@@ -352,7 +375,7 @@ def moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared=None) -> torch.Ten
     src = torch.empty(max(n, 1), dtype=torch.int32, device=dev)
     _call("dli_moe_align", _p(offsets), _p(pos), _p(src), _p(topk_ids), n, k, 0, E, _st())
     gu = grouped_linear_any(x, w_gu, offsets, src, n)
-    act = act_mul(gu, F2 // 2, x.dtype, "silu_mul", rows=offsets[E:])
+    act = act_mul(gu, F2 // 2, x.dtype, act, rows=offsets[E:], limit=limit)
     y = grouped_linear_any(act, w_down, offsets, None, n)
     ys = gate = None
     if shared is not None:
@@ -452,15 +475,16 @@ def side_gate(gate, ids, table, col0: int) -> torch.Tensor:
     return out
 
 
-def rmsnorm_cols(src, w, eps: float) -> torch.Tensor:
+def rmsnorm_cols(src, w, eps: float, gate=None) -> torch.Tensor:
     """RMS norm times w of the rows of an fp32 matrix that may be a column slice of a wider
-    one; storage dtype out."""
+    one, times sigmoid(gate) (fp32, same shape, may be a column slice) when given; storage
+    dtype out."""
     if not src.is_cuda:
-        return R.rmsnorm_cols(src, w, eps, w.dtype)
+        return R.rmsnorm_cols(src, w, eps, w.dtype, gate)
     T, n = src.shape
     out = torch.empty(T, n, dtype=w.dtype, device=src.device)
     _call("dli_rmsnorm_cols", _p(out), _p(src), src.stride(0), _p(w), T, n, float(eps),
-          _dt(w.dtype), _st())
+          _p(gate), gate.stride(0) if gate is not None else 0, _dt(w.dtype), _st())
     return out
 
 
@@ -555,4 +579,70 @@ def moe_gelu_experts_f32(x, w_up, w_down, topk_w, topk_ids, shared=None) -> torc
     out = torch.empty(T, D, dtype=torch.float32, device=dev)
     _call("dli_moe_combine_f32", _p(out), _p(y), None, _p(topk_w), _p(pos), _p(topk_ids), _p(x),
           x.stride(0), _p(ys), None, 0, T, k, D, E, _dt(x.dtype), _st())
+    return out
+
+
+# ----------------------------------------------------------------------------- hyper-connected designs
+def hyper_mix(xs, y, prev, read, w, eps: float = 0.0, w_offset: float = 0.0, dtype=None):
+    """One step of hyper-connections on the fp32 streams xs [T, S, D], in place
+    (``reference.hyper_mix``): with y (a sublayer's fp32 output) and ``prev`` (that sublayer's
+    fp32 vector read | write | mix) the streams are mixed and receive y; with ``read`` (the next
+    sublayer's vector, or ones for the plain sum) the weighted sum of the new streams is
+    returned — RMS-normed times (w + w_offset) in the storage dtype when w is given, else fp32."""
+    if not xs.is_cuda:
+        return R.hyper_mix(xs, y, prev, read, w, eps, w_offset, dtype or (w.dtype if w is not None else None))
+    T, S, D = xs.shape
+    h = None
+    if read is not None:
+        h = torch.empty(T, D, dtype=torch.float32 if w is None else w.dtype, device=xs.device)
+    _call("dli_hyper_mix", _p(xs), _p(y), y.stride(0) if y is not None else 0, _p(prev),
+          _p(read), _p(w), _p(h), T, S, D, float(eps), float(w_offset),
+          _dt(w.dtype) if w is not None else 1, _st())
+    return h
+
+
+def sink_prepare(proj, qw, kw, eps, H, G, d, dv, rot_dims, freq, mscale, positions, kcache,
+                 vcache, slots):
+    """Query / cache preparation of an attention whose q and k are RMS-normed over the whole
+    projection and partly rotated (``reference.sink_prepare``): k and v go to the cache rows,
+    the queries [T, H*d] come back in the storage dtype."""
+    dtype = qw.dtype
+    if not proj.is_cuda:
+        return R.sink_prepare(proj, qw, kw, eps, H, G, d, dv, rot_dims, freq, mscale, positions,
+                              kcache, vcache, slots, dtype)
+    T = proj.shape[0]
+    q = torch.empty(T, H * d, dtype=dtype, device=proj.device)
+    _call("dli_sink_prepare", _p(proj), proj.stride(0), _p(qw), _p(kw), float(eps), T, H, G, d,
+          dv, int(rot_dims), _p(freq), float(mscale), _p(positions), _p(q), _p(kcache),
+          _p(vcache), _p(slots), _dt(dtype), _st())
+    return q
+
+
+def lightning(proj, decays, state, slots, cu_seqlens, max_seqlen, positions, H, d, dv):
+    """Linear attention with one fixed decay per head over per-sequence state slots
+    (``reference.lightning``): the raw read-outs fp32 [T, H*dv]."""
+    if not proj.is_cuda:
+        return R.lightning(proj, decays, state, slots, cu_seqlens, positions, H, d, dv)
+    T = proj.shape[0]
+    S = cu_seqlens.shape[0] - 1
+    out = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
+    _call("dli_scalar_recurrence", _p(proj), proj.stride(0), 0, _p(decays), None, 0.0, None, 0.0,
+          _p(state), None, _p(slots), _p(cu_seqlens), _p(positions), _p(out), out.stride(0), 1.0,
+          S, int(max_seqlen), H, d, dv, 1, _st())
+    return out
+
+
+def mlstm(proj, if_b, cap: float, norm_w, eps: float, state, mstate, slots, cu_seqlens,
+          max_seqlen, positions, H, d, dv, out, out_scale: float = 1.0):
+    """Matrix memory with exponential gating over per-sequence state slots
+    (``reference.mlstm``); the normed, gated, scaled read-out is written to ``out`` [T, H*dv]
+    (storage dtype; may be a column slice of a wider buffer)."""
+    if not proj.is_cuda:
+        return R.mlstm(proj, if_b, cap, norm_w, eps, state, mstate, slots, cu_seqlens, positions,
+                       H, d, dv, out, out_scale)
+    S = cu_seqlens.shape[0] - 1
+    _call("dli_scalar_recurrence", _p(proj), proj.stride(0), 1, None, _p(if_b), float(cap),
+          _p(norm_w), float(eps), _p(state), _p(mstate), _p(slots), _p(cu_seqlens),
+          _p(positions), _p(out), out.stride(0), float(out_scale), S, int(max_seqlen), H, d, dv,
+          _dt(norm_w.dtype), _st())
     return out

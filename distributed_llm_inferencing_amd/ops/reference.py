@@ -385,19 +385,22 @@ def moe_mlp(x: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor,
 #   + offset), kv head g at columns ``[g*d, (g+1)*d)``
 # * recurrent state ``[state_slots, H, d, dv]`` fp32, one slot per live sequence
 def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
-                  out_dtype: torch.dtype) -> torch.Tensor:
+                  out_dtype: torch.dtype, w_offset: float = 0.0) -> torch.Tensor:
     """x fp32 [T, D] cut into ``groups`` equal parts, each divided by its own
     sqrt(mean(part^2) + eps); the whole times w."""
     T, D = x.shape
     xg = x.float().reshape(T, groups, D // groups)
     n = xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps)
-    return (n.reshape(T, D) * w.float()).to(out_dtype)
+    return (n.reshape(T, D) * (w.float() + w_offset)).to(out_dtype)
 
 
-def act_mul(gu: torch.Tensor, F_: int, out_dtype: torch.dtype, kind: str) -> torch.Tensor:
+def act_mul(gu: torch.Tensor, F_: int, out_dtype: torch.dtype, kind: str,
+            limit: float = 0.0) -> torch.Tensor:
     """The feed-forward's middle, fp32 in: ``gelu_mul`` / ``silu_mul`` = act(gu[:, :F]) *
     gu[:, F:2F]; ``gelu`` = gelu_tanh(gu[:, :F]); ``gelu_erf`` = the exact GELU of gu[:, :F];
     ``copy`` = gu[:, :F] itself."""
+    if kind == "clamp_swish":
+        return clamp_swish_mul(gu, F_, limit, out_dtype)
     g = gu[:, :F_].float()
     if kind == "gelu":
         return F.gelu(g, approximate="tanh").to(out_dtype)
@@ -465,14 +468,18 @@ def mla_prepare(proj, cw, eps, H, d, dr, r, rot_dims, inv_freq, positions, slots
 
 def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, positions, block_tables,
                      block_size, window, scale, slopes=None, talk=None, gate=None,
-                     out_dtype=None, chunk=0, k_groups=None):
+                     out_dtype=None, chunk=0, k_groups=None, sink=None, head_gate=False,
+                     out_scale=1.0):
     """q [T, H*dq]; k_cache rows [slots, G*dq]; v_cache rows [slots, >= G*dv] (may be k_cache:
     values = the first dv columns of each kv head's... row when G == 1). Every query at position
     p attends cached positions [max(0, p-window+1), p] of its sequence. fp32 softmax; ``talk``
     [H, H] mixes the heads' normalised weights; ``slopes`` [H] subtract slope*(p-j); ``gate``
     fp32 [T, H*dv] multiplies the output by its sigmoid. ``chunk`` > 0: only keys of the
     query's own block of ``chunk`` positions are visible. ``k_groups``: key heads per cache row
-    when it differs from the value heads G (1: every query head scores the whole key row)."""
+    when it differs from the value heads G (1: every query head scores the whole key row).
+    ``sink`` fp32 [H]: exp(sink_h) is added to head h's softmax denominator (a key without a
+    value). ``head_gate``: gate is fp32 [T, H], one number per head. ``out_scale`` multiplies
+    the output."""
     T = q.shape[0]
     Gk = G if k_groups is None else k_groups
     out = torch.zeros(T, H * dv, dtype=torch.float32, device=q.device)
@@ -499,14 +506,23 @@ def window_attention(q, k_cache, v_cache, dq, dv, H, G, cu_seqlens, positions, b
         if chunk:
             vis = vis & ((pos[:, None] // chunk) == (j[None, :] // chunk))
         sc = sc.masked_fill(~vis[None], float("-inf"))
-        w = torch.softmax(sc, dim=-1)
+        if sink is not None:
+            n = sc.shape[1]
+            sc = torch.cat([sc, sink.float()[:, None, None].expand(H, n, 1)], -1)
+            w = torch.softmax(sc, dim=-1)[..., :-1]
+        else:
+            w = torch.softmax(sc, dim=-1)
         if talk is not None:
             w = torch.einsum("hg,gtj->htj", talk.float(), w)
         ve = vv.repeat_interleave(rep, dim=1)                                   # [ctx, H, dv]
         o = torch.einsum("htj,jhd->thd", w, ve)
         out[t0:t1] = o.reshape(t1 - t0, H * dv)
-    if gate is not None:
+    if gate is not None and head_gate:
+        out = (out.reshape(T, H, dv) * torch.sigmoid(gate.float())[:, :, None]).reshape(T, H * dv)
+    elif gate is not None:
         out = out * torch.sigmoid(gate.float())
+    if out_scale != 1.0:
+        out = out * out_scale
     return out.to(out_dtype or q.dtype)
 
 
@@ -599,7 +615,7 @@ def score_router(h, w_router, correction, top, n_gate=0):
     return sc.gather(1, ids), ids.to(torch.int32), torch.sigmoid(z[:, n:])
 
 
-def moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared=None):
+def moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared=None, act="silu_mul", limit=0.0):
     """Weighted sum of each token's chosen experts, fp32 out. Expert e < E (w_gu [E, 2F, D] =
     gate | up, w_down [E, D, F]) is down(silu(gate) * up); ids >= E are identity experts (the
     input itself). ``shared`` = (ws_gu, ws_down, gate [T]) adds an always-on expert times its
@@ -611,7 +627,7 @@ def moe_experts_f32(x, w_gu, w_down, topk_w, topk_ids, shared=None):
         rows, slot = (topk_ids == e).nonzero(as_tuple=True)
         if rows.numel() == 0:
             continue
-        a = act_mul(linear(x[rows], w_gu[e], out_dtype=torch.float32), F2 // 2, x.dtype, "silu_mul")
+        a = act_mul(linear(x[rows], w_gu[e], out_dtype=torch.float32), F2 // 2, x.dtype, act, limit)
         y = linear(a, w_down[e], out_dtype=torch.float32)
         out.index_add_(0, rows, y * topk_w[rows, slot][:, None])
     wi = (topk_w * (topk_ids >= E)).sum(-1, keepdim=True)
@@ -685,10 +701,14 @@ def side_gate(gate, ids, table, col0, out_dtype):
     return (F.gelu(gate.float(), approximate="tanh") * e).to(out_dtype)
 
 
-def rmsnorm_cols(src, w, eps, out_dtype):
-    """Rows of the fp32 (column-sliced) matrix ``src`` divided by their RMS, times w."""
+def rmsnorm_cols(src, w, eps, out_dtype, gate=None):
+    """Rows of the fp32 (column-sliced) matrix ``src`` divided by their RMS, times w (and times
+    sigmoid(gate), an fp32 matrix of the same shape, when given)."""
     v = src.float()
-    return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+    o = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    if gate is not None:
+        o = o * torch.sigmoid(gate.float())
+    return o.to(out_dtype)
 
 
 def rotate_pairs(x, positions, inv_freq, rot_dims, half):
@@ -790,3 +810,160 @@ def moe_gelu_experts_f32(x, w_up, w_down, topk_w, topk_ids, shared=None):
         a = F.gelu(linear(x, shared[0], out_dtype=torch.float32)).to(x.dtype)
         out += linear(a, shared[1], out_dtype=torch.float32)
     return out
+
+
+# ----------------------------------------------------------------------------- hyper-connected designs
+def hyper_mix(xs, y, prev, read, w, eps, w_offset, out_dtype):
+    """Hyper-connections over xs fp32 [T, S, D] (in place). ``prev`` / ``read`` are fp32
+    vectors [S + S + S*S] = read weights | write weights | stream mix [from, to] of the
+    sublayer that produced y and of the one that runs next. With y: every stream becomes
+    xs[:, t] = sum_s mix[s, t] xs[:, s] + write[t] * y. With ``read``: u = sum_s read[s] xs[:, s]
+    is returned, RMS-normed times (w + w_offset) in ``out_dtype`` when w is given, else as
+    fp32."""
+    T, S, D = xs.shape
+    if y is not None:
+        mix = prev[2 * S:].reshape(S, S).float()
+        new = torch.einsum("sr,tsd->trd", mix, xs) + prev[S:2 * S].float()[None, :, None] * y.float()[:, None, :]
+        xs.copy_(new)
+    if read is None:
+        return None
+    u = torch.einsum("s,tsd->td", read[:S].float(), xs)
+    if w is None:
+        return u
+    h = u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * (w.float() + w_offset)
+    return h.to(out_dtype)
+
+
+def sink_prepare(proj, qw, kw, eps, H, G, d, dv, rot_dims, freq, mscale, positions, kcache,
+                 vcache, slots, out_dtype):
+    """proj fp32 [T, >= H*d + G*d + G*dv] = [q | k | v | ...]: q and k are RMS-normed over their
+    whole rows (all heads at once) times qw / kw, then the first rot_dims dims of every head
+    rotate (dimension i with i + rot_dims/2) by positions * freq (float64) with cos and sin
+    times mscale; k and v go to the cache rows; returns q [T, H*d]."""
+    T = proj.shape[0]
+    q = proj[:, :H * d].float()
+    k = proj[:, H * d:(H + G) * d].float()
+    v = proj[:, (H + G) * d:(H + G) * d + G * dv].float()
+    q = (q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qw.float()).reshape(T, H, d)
+    k = (k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * kw.float()).reshape(T, G, d)
+    if rot_dims:
+        hh = rot_dims // 2
+        ang = positions.double()[:, None] * freq.double()[None, :]
+        c = (ang.cos() * mscale).float()[:, None, :]
+        s = (ang.sin() * mscale).float()[:, None, :]
+
+        def rot(x):
+            o = x.clone()
+            a, b = x[..., :hh], x[..., hh:rot_dims]
+            o[..., :hh] = a * c - b * s
+            o[..., hh:rot_dims] = b * c + a * s
+            return o
+        q, k = rot(q), rot(k)
+    ok = slots >= 0
+    idx = slots[ok].long()
+    kcache[idx] = k.reshape(T, G * d)[ok].to(kcache.dtype)
+    vcache[idx] = v[ok].to(vcache.dtype)
+    return q.reshape(T, H * d).to(out_dtype)
+
+
+def lightning(proj, decays, state, slots, cu_seqlens, positions, H, d, dv):
+    """Linear attention with a fixed decay per head. proj fp32 [T, 2*H*d + H*dv (+ ...)] = [q |
+    k | v | ...] before their SiLU; per head S = decay_h S + k v^T, o = S^T q; returns the raw
+    read-outs fp32 [T, H*dv]. state fp32 [slots, H, d, dv] in place; a portion whose first
+    position is 0 starts from zero."""
+    T = proj.shape[0]
+    out = torch.zeros(T, H * dv, dtype=torch.float32, device=proj.device)
+    cu, sl = cu_seqlens.tolist(), slots.tolist()
+    a = decays.float().reshape(H, 1, 1)
+    for s in range(len(cu) - 1):
+        t0, t1 = cu[s], cu[s + 1]
+        if t1 <= t0 or sl[s] < 0:
+            continue
+        S = state[sl[s]].clone()
+        if int(positions[t0]) == 0:
+            S.zero_()
+        p = F.silu(proj[t0:t1, :2 * H * d + H * dv].float())
+        qv = p[:, :H * d].reshape(-1, H, d)
+        kv = p[:, H * d:2 * H * d].reshape(-1, H, d)
+        vv = p[:, 2 * H * d:].reshape(-1, H, dv)
+        for t in range(t1 - t0):
+            S = a * S + kv[t][:, :, None] * vv[t][:, None, :]
+            out[t0 + t] = torch.einsum("hdv,hd->hv", S, qv[t]).reshape(H * dv)
+        state[sl[s]] = S
+    return out
+
+
+def mlstm(proj, if_b, cap, norm_w, eps, state, mstate, slots, cu_seqlens, positions, H, d, dv,
+          out, out_scale):
+    """Matrix memory with exponential gating. proj fp32 [T, 2*H*d + 2*H*dv + 2*H] = [q | k | v |
+    output gate | input gates | forget gates]. Per head, with i = cap tanh((z_i + b_i) / cap),
+    f = logsigmoid(cap tanh((z_f + b_f) / cap)) and a running maximum m (0 at the start):
+        m' = max(f + m, i);  S = e^(f + m - m') S + e^(i - m') k v^T;  n likewise with k alone;
+        o = S^T q d^(-1/2) / (max(|n . q d^(-1/2)|, e^(-m')) + 1e-6)
+    o is RMS-normed per head, times norm_w [H*dv], sigmoid(gate) and out_scale, and written to
+    ``out`` [T, H*dv]. state fp32 [slots, H, d, dv + 1] holds S and, as its last column, n;
+    mstate fp32 [slots, H] holds m."""
+    T = proj.shape[0]
+    cu, sl = cu_seqlens.tolist(), slots.tolist()
+    nw = norm_w.float().reshape(H, dv)
+    o0 = 2 * H * d
+    for s in range(len(cu) - 1):
+        t0, t1 = cu[s], cu[s + 1]
+        if t1 <= t0:
+            continue
+        if sl[s] < 0:
+            out[t0:t1] = 0
+            continue
+        S = state[sl[s]].clone()
+        m = mstate[sl[s]].clone()
+        if int(positions[t0]) == 0:
+            S.zero_()
+            m.zero_()
+        p = proj[t0:t1].float()
+        qv = p[:, :H * d].reshape(-1, H, d) * (d ** -0.5)
+        kv = p[:, H * d:o0].reshape(-1, H, d)
+        vv = p[:, o0:o0 + H * dv].reshape(-1, H, dv)
+        gv = p[:, o0 + H * dv:o0 + 2 * H * dv].reshape(-1, H, dv)
+        b = if_b.float()
+        ig = cap * torch.tanh((p[:, o0 + 2 * H * dv:o0 + 2 * H * dv + H] + b[:H]) / cap)
+        fg = F.logsigmoid(cap * torch.tanh((p[:, o0 + 2 * H * dv + H:o0 + 2 * H * dv + 2 * H]
+                                            + b[H:]) / cap))
+        ones = torch.ones(H, 1, dtype=torch.float32, device=proj.device)
+        for t in range(t1 - t0):
+            m1 = torch.maximum(fg[t] + m, ig[t])
+            a, bb = torch.exp(fg[t] + m - m1), torch.exp(ig[t] - m1)
+            v1 = torch.cat([vv[t], ones], 1)
+            S = a[:, None, None] * S + bb[:, None, None] * kv[t][:, :, None] * v1[:, None, :]
+            m = m1
+            r = torch.einsum("hdv,hd->hv", S, qv[t])
+            o = r[:, :dv] / (torch.maximum(r[:, dv:].abs(), torch.exp(-m)[:, None]) + 1e-6)
+            o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * nw
+            out[t0 + t] = (o * torch.sigmoid(gv[t]) * out_scale).reshape(H * dv).to(out.dtype)
+        state[sl[s]] = S
+        mstate[sl[s]] = m
+    return out
+
+
+def group_router(h, w_router, top, groups, keep, wscale):
+    """Router over groups of neighbouring experts: s = softmax of the fp32 logits h @ w^T over
+    all experts; a group scores its best expert; only experts of the ``keep`` best of
+    ``groups`` equal groups can be chosen; the ``top`` largest s among them are chosen (lowest
+    index on ties) with weights s * wscale (not renormalised). Returns (weights fp32 [T, top],
+    ids int32 [T, top])."""
+    z = h.float() @ w_router.float().t()
+    s = torch.softmax(z, -1)
+    T, E = s.shape
+    gs = s.reshape(T, groups, E // groups).max(-1).values
+    order = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep]
+    allowed = torch.zeros(T, groups, dtype=torch.bool, device=h.device)
+    allowed.scatter_(1, order, True)
+    masked = torch.where(allowed.repeat_interleave(E // groups, dim=1), s, torch.full_like(s, -1.0))
+    ids = torch.sort(masked, dim=-1, descending=True, stable=True).indices[:, :top]
+    return s.gather(1, ids) * wscale, ids.to(torch.int32)
+
+
+def clamp_swish_mul(gu, F_, limit, out_dtype):
+    """g = min(gu[:, :F], limit), u = clamp(gu[:, F:2F], -limit, limit): g sigmoid(1.702 g) (u + 1)."""
+    g = gu[:, :F_].float().clamp(max=limit)
+    u = gu[:, F_:2 * F_].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(out_dtype)
