@@ -62,7 +62,7 @@ __global__ void __launch_bounds__(256) resadd_groupnorm_kernel(
     float* __restrict__ x, const float* __restrict__ y, int ldy, const S* __restrict__ bias,
     float keep, float mult, const S* __restrict__ w, void* __restrict__ h, int ldh, int dim,
     int groups, float eps, const long* __restrict__ rows_idx, bool vec4, float gain,
-    bool h_f32) {
+    bool h_f32, float w_offset) {
   extern __shared__ __attribute__((aligned(16))) float row[];   // dim floats + group scales
   float* gsum = row + dim;
   const int r = blockIdx.x;
@@ -111,10 +111,10 @@ __global__ void __launch_bounds__(256) resadd_groupnorm_kernel(
   __syncthreads();
   if (h_f32) {
     for (int c = threadIdx.x; c < dim; c += blockDim.x)
-      ((float*)h)[(long)r * ldh + c] = row[c] * gsum[c / gl] * ldf(w + c) * gain;
+      ((float*)h)[(long)r * ldh + c] = row[c] * gsum[c / gl] * (ldf(w + c) + w_offset) * gain;
   } else {
     for (int c = threadIdx.x; c < dim; c += blockDim.x)
-      stf((S*)h + (long)r * ldh + c, row[c] * gsum[c / gl] * ldf(w + c) * gain);
+      stf((S*)h + (long)r * ldh + c, row[c] * gsum[c / gl] * (ldf(w + c) + w_offset) * gain);
   }
 }
 
@@ -183,7 +183,12 @@ __device__ __forceinline__ float gelu_tanh32(float z) {
   return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
-__device__ __forceinline__ float act_pair(int kind, float g, float u) {
+__device__ __forceinline__ float act_pair(int kind, float g, float u, float limit) {
+  if (kind == 5) {                       // clamped swish: min / clamp, then g sigmoid(1.702 g) (u + 1)
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+  }
   if (kind == 0) return gelu_tanh32(g) * u;
   if (kind == 1) return g / (1.f + expf(-g)) * u;
   if (kind == 3) return 0.5f * g * (1.f + erff(g * 0.7071067811865476f));
@@ -192,25 +197,27 @@ __device__ __forceinline__ float act_pair(int kind, float g, float u) {
 }
 
 // kind 0: gelu_tanh(gu[:, c]) * gu[:, F + c]; 1: silu(..) * ..; 2: gelu_tanh(gu[:, c]);
-// 3: the exact (erf) GELU of gu[:, c]; 4: gu[:, c] itself (a rounding copy of a column slice).
+// 3: the exact (erf) GELU of gu[:, c]; 4: gu[:, c] itself (a rounding copy of a column slice);
+// 5: g sigmoid(1.702 g) (u + 1) with g = min(gu[:, c], limit), u = clamp(gu[:, F + c], +-limit).
 // nrows (nullable, device): rows from *nrows on hold no data and are skipped.
 template <typename S>
 __global__ void __launch_bounds__(256) act_mul_kernel(
     S* __restrict__ out, int ldo, const float* __restrict__ gu, int ldg, int T, int F, int kind,
-    const int* __restrict__ nrows) {
+    const int* __restrict__ nrows, float limit) {
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid >= (long)T * F) return;
   const int t = (int)(gid / F), c = (int)(gid % F);
   if (nrows != nullptr && t >= *nrows) return;
   const float* r = gu + (long)t * ldg;
-  stf(out + (long)t * ldo + c, act_pair(kind, r[c], kind >= 2 ? 0.f : r[F + c]));
+  stf(out + (long)t * ldo + c,
+      act_pair(kind, r[c], (kind >= 2 && kind != 5) ? 0.f : r[F + c], limit));
 }
 
 // 4 features a thread (F, ldg multiples of 4, 16-byte aligned rows): 16-byte loads
 template <typename S>
 __global__ void __launch_bounds__(256) act_mul4_kernel(
     S* __restrict__ out, int ldo, const float* __restrict__ gu, int ldg, int T, int F, int kind,
-    const int* __restrict__ nrows) {
+    const int* __restrict__ nrows, float limit) {
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const int f4 = F >> 2;
   if (gid >= (long)T * f4) return;
@@ -219,9 +226,10 @@ __global__ void __launch_bounds__(256) act_mul4_kernel(
   const float* r = gu + (long)t * ldg;
   const f32x4 g = *reinterpret_cast<const f32x4*>(r + c);
   f32x4 u = f32x4{0.f, 0.f, 0.f, 0.f};
-  if (kind < 2) u = *reinterpret_cast<const f32x4*>(r + F + c);
+  if (kind < 2 || kind == 5) u = *reinterpret_cast<const f32x4*>(r + F + c);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) stf(out + (long)t * ldo + c + i, act_pair(kind, g[i], u[i]));
+  for (int i = 0; i < 4; ++i)
+    stf(out + (long)t * ldo + c + i, act_pair(kind, g[i], u[i], limit));
 }
 
 // Grid (token, head slices). proj row (fp32, + bias): [H*d q | G*d k | G*dv v] (q only when the
@@ -407,8 +415,8 @@ extern "C" int dli_embedding_f32(float* x, float* x0, const int* ids, const void
 extern "C" int dli_resadd_groupnorm(float* x, const float* y, int ldy, const void* bias,
                                     float keep, float mult, const void* w, void* h, int ldh,
                                     int rows, int dim, int groups, float eps,
-                                    const long* rows_idx, float gain, int h_f32, int dt,
-                                    hipStream_t st) {
+                                    const long* rows_idx, float gain, int h_f32, float w_offset,
+                                    int dt, hipStream_t st) {
   if (rows <= 0) return 0;
   if (groups < 1 || dim % groups || (size_t)(dim + groups) * 4 > 60000)
     return (int)hipErrorInvalidValue;
@@ -418,10 +426,10 @@ extern "C" int dli_resadd_groupnorm(float* x, const float* y, int ldy, const voi
   DT_SWITCH(dt,
             (resadd_groupnorm_kernel<u16><<<rows, 256, sh, st>>>(
                 x, y, ldy, (const u16*)bias, keep, mult, (const u16*)w, h, ldh, dim, groups,
-                eps, rows_idx, vec4, gain, h_f32 != 0)),
+                eps, rows_idx, vec4, gain, h_f32 != 0, w_offset)),
             (resadd_groupnorm_kernel<float><<<rows, 256, sh, st>>>(
                 x, y, ldy, (const float*)bias, keep, mult, (const float*)w, h, ldh, dim,
-                groups, eps, rows_idx, vec4, gain, h_f32 != 0)));
+                groups, eps, rows_idx, vec4, gain, h_f32 != 0, w_offset)));
   DLI_RETURN_LAUNCH();
 }
 
@@ -452,19 +460,19 @@ extern "C" int dli_token_shift(const float* h, const void* mu, float* state, con
 }
 
 extern "C" int dli_act_mul(void* out, int ldo, const float* gu, int ldg, int T, int F, int kind,
-                           const int* nrows, int dt, hipStream_t st) {
+                           const int* nrows, float limit, int dt, hipStream_t st) {
   if (T <= 0) return 0;
-  if (kind < 0 || kind > 4) return (int)hipErrorInvalidValue;
+  if (kind < 0 || kind > 5) return (int)hipErrorInvalidValue;
   if (F % 4 == 0 && ldg % 4 == 0 && (uintptr_t)gu % 16 == 0) {
     const int nb4 = (int)(((long)T * (F / 4) + 255) / 256);
     DT_SWITCH(dt,
-              (act_mul4_kernel<u16><<<nb4, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F, kind, nrows)),
-              (act_mul4_kernel<float><<<nb4, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F, kind, nrows)));
+              (act_mul4_kernel<u16><<<nb4, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F, kind, nrows, limit)),
+              (act_mul4_kernel<float><<<nb4, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F, kind, nrows, limit)));
     DLI_RETURN_LAUNCH();
   }
   const int nb = (int)(((long)T * F + 255) / 256);
-  DT_SWITCH(dt, (act_mul_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F, kind, nrows)),
-            (act_mul_kernel<float><<<nb, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F, kind, nrows)));
+  DT_SWITCH(dt, (act_mul_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F, kind, nrows, limit)),
+            (act_mul_kernel<float><<<nb, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F, kind, nrows, limit)));
   DLI_RETURN_LAUNCH();
 }
 

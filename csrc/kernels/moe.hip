@@ -430,7 +430,7 @@ template <typename S>
 __global__ void __launch_bounds__(256) score_router_kernel(
     float* __restrict__ topk_w, int* __restrict__ topk_ids, float* __restrict__ gates,
     const S* __restrict__ h, int ldh, const S* __restrict__ W, const float* __restrict__ corr,
-    int D, int n, int n_gate, int top, bool vec) {
+    int D, int n, int n_gate, int top, bool vec, int groups, int keep, float wscale) {
   extern __shared__ __attribute__((aligned(16))) float rsm[];                      // [D] row, [n + n_gate] logits
   float* row = rsm;
   float* z = rsm + D;
@@ -486,19 +486,40 @@ __global__ void __launch_bounds__(256) score_router_kernel(
   for (int e = 0; e < n; ++e) { const float v = expf(z[e] - m); z[e] = v; sum += v; }
   const float inv = 1.f / sum;
   for (int g = 0; g < n_gate; ++g) gates[(long)t * n_gate + g] = 1.f / (1.f + expf(-z[n + g]));
+  // groups of n / groups neighbours: a group scores its best expert; the experts of all but
+  // the `keep` best groups (lowest index on ties) leave the choice (their slot marked -2)
+  if (groups > 1 && keep < groups) {
+    const int gl = n / groups;
+    float* gs = z + n + n_gate;                    // [groups]
+    for (int g = 0; g < groups; ++g) {
+      float b = 0.f;
+      for (int e = g * gl; e < (g + 1) * gl; ++e) b = fmaxf(b, z[e]);
+      gs[g] = b;
+    }
+    for (int j = 0; j < keep; ++j) {
+      int best = -1;
+      for (int g = 0; g < groups; ++g)
+        if (gs[g] >= 0.f && (best < 0 || gs[g] > gs[best])) best = g;
+      gs[best] = -1.f;                               // kept
+    }
+    for (int g = 0; g < groups; ++g)
+      if (gs[g] >= 0.f)
+        for (int e = g * gl; e < (g + 1) * gl; ++e) z[e] = -2.f;
+  }
   // selection rounds; a chosen expert's score is kept aside and its slot marked with -2
   for (int j = 0; j < top; ++j) {
     int best = -1;
-    float bc = -INFINITY;
+    float bc = -INFINITY, bz = 0.f;
     for (int e = 0; e < n; ++e) {
       const float sc = z[e];
       if (sc == -2.f) continue;
-      const float c = sc * inv + corr[e];
-      if (best < 0 || c > bc) { best = e; bc = c; }
+      const float c = sc * inv + (corr != nullptr ? corr[e] : 0.f);
+      if (best < 0 || c > bc) { best = e; bc = c; bz = sc; }
     }
+    if (best < 0) { best = 0; bz = 0.f; }            // fewer candidates than `top`: weight 0
     topk_ids[(long)t * top + j] = best;
-    topk_w[(long)t * top + j] = z[best] * inv;
-    z[best] = -2.f;
+    topk_w[(long)t * top + j] = bz * inv * wscale;
+    if (z[best] != -2.f) z[best] = -2.f;
   }
 }
 
@@ -532,19 +553,22 @@ __global__ void __launch_bounds__(256) moe_combine_f32_kernel(
 
 extern "C" int dli_score_router(float* topk_w, int* topk_ids, float* gates, const void* h, int ldh,
                                 const void* W, const float* corr, int T, int D, int n, int n_gate,
-                                int top, int dt, hipStream_t st) {
+                                int top, int groups, int keep, float wscale, int dt,
+                                hipStream_t st) {
   if (T <= 0) return 0;
-  if (n < 1 || n_gate < 0 || top < 1 || top > n || n + n_gate > ROUTER_MAX ||
-      (size_t)(D + n + n_gate) * 4 > 60000)
+  if (n < 1 || n_gate < 0 || top < 1 || top > n || n + n_gate > ROUTER_MAX || groups < 1 ||
+      n % groups || keep < 1 || keep > groups || (size_t)(D + n + n_gate + groups) * 4 > 60000)
     return (int)hipErrorInvalidValue;
-  const size_t sh = (size_t)(D + n + n_gate) * 4;
+  const size_t sh = (size_t)(D + n + n_gate + groups) * 4;
   const bool vec = (uintptr_t)W % 16 == 0 && D % (dt == 0 ? 8 : 4) == 0;
   if (dt == 0)
     score_router_kernel<u16><<<T, 256, sh, st>>>(topk_w, topk_ids, gates, (const u16*)h, ldh,
-                                                 (const u16*)W, corr, D, n, n_gate, top, vec);
+                                                 (const u16*)W, corr, D, n, n_gate, top, vec,
+                                                 groups, keep, wscale);
   else if (dt == 1)
     score_router_kernel<float><<<T, 256, sh, st>>>(topk_w, topk_ids, gates, (const float*)h, ldh,
-                                                   (const float*)W, corr, D, n, n_gate, top, vec);
+                                                   (const float*)W, corr, D, n, n_gate, top, vec,
+                                                   groups, keep, wscale);
   else return (int)hipErrorInvalidValue;
   DLI_RETURN_LAUNCH();
 }

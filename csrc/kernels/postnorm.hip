@@ -12,7 +12,7 @@
 //  * add_rmsnormed     x += y / sqrt(mean(y^2) + eps) * w in place, and the S copy of x
 //  * side_gate         gelu_tanh(gate) * table[id, col0 + c] -> S (a per-layer slice of a
 //                      second embedding table gates a small projection)
-//  * rmsnorm_cols      RMS norm * w of a column slice of an fp32 projection -> S
+//  * rmsnorm_cols      RMS norm * w (* sigmoid(gate)) of a column slice of an fp32 projection -> S
 //  * latent_prepare    latent attention with the queries and the compressed kv in separate
 //                      projections: RMS norm of the latent -> cache, rotary on the shared key ->
 //                      cache (skipped by a layer that reads another layer's cache), rotary on
@@ -205,7 +205,7 @@ __global__ void __launch_bounds__(256) side_gate_kernel(
 template <typename S>
 __global__ void __launch_bounds__(256) rmsnorm_cols_kernel(
     S* __restrict__ out, const float* __restrict__ src, int lds, const S* __restrict__ w, int T,
-    int n, float eps, bool vec4) {
+    int n, float eps, bool vec4, const float* __restrict__ gate, int ldg) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (t >= T) return;
@@ -218,14 +218,25 @@ __global__ void __launch_bounds__(256) rmsnorm_cols_kernel(
     }
     s = wave_sum(s);
     const float rs = 1.f / sqrtf(s / (float)n + eps);
-    for (int c = lane * 4; c < n; c += 256)
-      st4(out + (long)t * n + c, *reinterpret_cast<const f32x4*>(r + c) * rs * ld4(w + c));
+    for (int c = lane * 4; c < n; c += 256) {
+      f32x4 v = *reinterpret_cast<const f32x4*>(r + c) * rs * ld4(w + c);
+      if (gate != nullptr) {
+        const f32x4 g = *reinterpret_cast<const f32x4*>(gate + (long)t * ldg + c);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] *= 1.f / (1.f + expf(-g[u]));
+      }
+      st4(out + (long)t * n + c, v);
+    }
     return;
   }
   for (int c = lane; c < n; c += 64) { const float v = r[c]; s += v * v; }
   s = wave_sum(s);
   const float rs = 1.f / sqrtf(s / (float)n + eps);
-  for (int c = lane; c < n; c += 64) stf(out + (long)t * n + c, r[c] * rs * ldf(w + c));
+  for (int c = lane; c < n; c += 64) {
+    float v = r[c] * rs * ldf(w + c);
+    if (gate != nullptr) v *= 1.f / (1.f + expf(-gate[(long)t * ldg + c]));
+    stf(out + (long)t * n + c, v);
+  }
 }
 
 // The rotation of element c of a rotated part `v` (length >= rot_dims): with `half` dimension
@@ -461,17 +472,18 @@ extern "C" int dli_side_gate(void* out, const float* gate, int ldg, const int* i
 }
 
 extern "C" int dli_rmsnorm_cols(void* out, const float* src, int lds, const void* w, int T, int n,
-                                float eps, int dt, hipStream_t st) {
+                                float eps, const float* gate, int ldg, int dt, hipStream_t st) {
   if (T <= 0) return 0;
   if (n < 1) return (int)hipErrorInvalidValue;
   const int nb = (T + 3) / 4;
-  const bool vec4 = n % 4 == 0 && lds % 4 == 0 &&
-                    (((uintptr_t)out | (uintptr_t)src | (uintptr_t)w) & 15) == 0;
+  const bool vec4 = n % 4 == 0 && lds % 4 == 0 && ldg % 4 == 0 &&
+                    (((uintptr_t)out | (uintptr_t)src | (uintptr_t)w | (uintptr_t)gate) & 15) == 0;
   DT_SWITCH(dt,
             (rmsnorm_cols_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, src, lds, (const u16*)w, T,
-                                                          n, eps, vec4)),
+                                                          n, eps, vec4, gate, ldg)),
             (rmsnorm_cols_kernel<float><<<nb, 256, 0, st>>>((float*)out, src, lds,
-                                                            (const float*)w, T, n, eps, vec4)));
+                                                            (const float*)w, T, n, eps, vec4,
+                                                            gate, ldg)));
   DLI_RETURN_LAUNCH();
 }
 

@@ -10,7 +10,11 @@
 //                     own key/value head. Needs the normalised weights of every head, so the
 //                     kernel makes two passes over the window: (1) running max / sum per head,
 //                     (2) weights, mix, weighted value sum.
-//  * gate    != null: out *= sigmoid(gate) (fp32 pre-activation of the same token, ldg)
+//  * gate    != null: out *= sigmoid(gate) (fp32 pre-activation of the same token, ldg); with
+//                     head_gate the gate row holds one number per head
+//  * sink    != null: exp(sink[h]) joins head h's softmax denominator: a key with that score
+//                     and no value, counted once (the running max / sum start from it)
+//  * out_scale:       the output is multiplied by it
 //  * chunk   > 0: a query also sees only the keys of its own block of `chunk` positions
 //                     (blocks counted from position 0 of the sequence)
 //  * Gk != G: the key rows hold Gk heads of dq while the values hold G heads of dv (Gk = 1:
@@ -53,6 +57,8 @@ struct WinAttnArgs {
   int H, G, dq, dv, window;
   float scale;
   int Gk, chunk;
+  const float* sink;                    // [H] or null
+  int head_gate; float out_scale;
 };
 
 template <typename S>
@@ -75,7 +81,10 @@ __global__ void __launch_bounds__(256) window_attention_kernel(WinAttnArgs a) {
   const int tid = threadIdx.x;
   const S* qrow = (const S*)a.q + (long)t * a.ldq;
   for (int i = tid; i < H * dq; i += blockDim.x) qs[i] = ldf(qrow + i);
-  for (int h = tid; h < H; h += blockDim.x) { hm[h] = -INFINITY; hl[h] = 0.f; }
+  for (int h = tid; h < H; h += blockDim.x) {
+    hm[h] = a.sink != nullptr ? a.sink[h] : -INFINITY;
+    hl[h] = a.sink != nullptr ? 1.f : 0.f;
+  }
   const int* bt = a.block_tables + (long)s * a.bt_stride;
   const int hpg = H / G, hpk = H / a.Gk;
   float acc[MAX_ACC];
@@ -161,8 +170,9 @@ __global__ void __launch_bounds__(256) window_attention_kernel(WinAttnArgs a) {
     const int o = tid + i * 256;
     if (o < H * dv) {
       float v = acc[i];
-      if (a.gate != nullptr) v *= 1.f / (1.f + expf(-a.gate[(long)t * a.ldg + o]));
-      stf(orow + o, v);
+      if (a.gate != nullptr)
+        v *= 1.f / (1.f + expf(-a.gate[(long)t * a.ldg + (a.head_gate ? o / dv : o)]));
+      stf(orow + o, v * a.out_scale);
     }
   }
 }
@@ -174,7 +184,7 @@ extern "C" int dli_window_attention(
     int ldo, const float* gate, int ldg, const float* slopes, const float* talk, const int* cu,
     const int* positions, const int* block_tables, int bt_stride, int block_size, int num_seqs,
     int max_seqlen, int H, int G, int dq, int dv, int window, float scale, int Gk, int chunk,
-    int dt, hipStream_t st) {
+    const float* sink, int head_gate, float out_scale, int dt, hipStream_t st) {
   if (num_seqs <= 0 || max_seqlen <= 0) return 0;
   if (H < 1 || G < 1 || H % G || Gk < 1 || H % Gk || chunk < 0 || dq < 1 || dv < 1 ||
       window < 1 || block_size < 1 ||
@@ -195,7 +205,7 @@ extern "C" int dli_window_attention(
   }
   WinAttnArgs a{q, ldq, k, k_stride, v, v_stride, out, ldo, gate, ldg, slopes, talk, cu,
                 positions, block_tables, bt_stride, block_size, H, G, dq, dv, window, scale,
-                Gk, chunk};
+                Gk, chunk, sink, head_gate, out_scale};
   dim3 grid(max_seqlen, num_seqs);
   if (dt == 0) window_attention_kernel<u16><<<grid, 256, sh, st>>>(a);
   else if (dt == 1) window_attention_kernel<float><<<grid, 256, sh, st>>>(a);

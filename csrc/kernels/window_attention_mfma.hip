@@ -630,9 +630,11 @@ extern "C" int dli_window_attention_mfma(
     int ldo, const float* gate, int ldg, const float* slopes, const float* talk, const int* cu,
     const int* positions, const int* block_tables, int bt_stride, int block_size, int num_seqs,
     int max_seqlen, int H, int G, int dq, int dv, int window, float scale, int T, void* ws,
-    int rowhead, int Gk, int chunk, hipStream_t st) {
+    int rowhead, int Gk, int chunk, const float* sink, int head_gate, float out_scale,
+    hipStream_t st) {
   if (num_seqs <= 0 || max_seqlen <= 0) return 0;
   if (chunk < 0 || Gk < 1) return (int)hipErrorInvalidValue;
+  if (sink != nullptr || head_gate || out_scale != 1.f) return (int)hipErrorNotSupported;
   // keys a query tile can see: bounds the slot table and the key splits
   const int weff = chunk > 0 && chunk < window ? chunk : window;
   int rowmul = 1, vrows = 0;
