@@ -254,3 +254,72 @@ def route_margins(c, w, tokens):
             else:
                 x = x + y
     return best
+
+
+# ----------------------------------------------------------------------------- test weights
+def bf16_exact(a):
+    """Round to values bfloat16 holds exactly (so that every precision sees the same weights)."""
+    import torch
+    return torch.as_tensor(np.asarray(a, np.float64)).to(torch.bfloat16).double().numpy()
+
+
+def random_weights(c, seed=0):
+    """Checkpoint-named float64 arrays (bfloat16-exact) for configuration ``c``."""
+    rng = np.random.default_rng(seed)
+    D, V = int(c["width"]), int(c["vocab"])
+    ns = int(c.get("streams") or 0)
+    w = {}
+
+    def lin(name, o, i, gain=1.0):
+        w[name] = rng.standard_normal((o, i)) * gain / math.sqrt(i)
+
+    w["embed"] = rng.standard_normal((V, D)) * 0.5
+    lin("head", V, D)
+    w["final.norm"] = rng.standard_normal(D) * 0.2
+    for i, L in enumerate(c["layers"]):
+        a, mx = f"l{i}.", L["mixer"]
+        for q in (1, 2):
+            if q == 2 and not L.get("mlp"):
+                continue
+            w[f"{a}norm{q}"] = rng.standard_normal(D) * 0.2
+            if ns:
+                w[f"{a}hc{q}.in"] = 1.0 / ns + 0.2 * rng.standard_normal(ns)
+                w[f"{a}hc{q}.out"] = 1.0 + 0.3 * rng.standard_normal(ns)
+                w[f"{a}hc{q}.mix"] = np.eye(ns) + 0.2 * rng.standard_normal((ns, ns))
+        m = a + "mix."
+        if L["type"] == "lightning":
+            H, d, dv = int(mx["heads"]), int(mx["dim"]), int(mx["vdim"])
+            lin(m + "q", H * d, D, 2.0), lin(m + "k", H * d, D, 2.0)
+            lin(m + "v", H * dv, D, 2.0), lin(m + "g", H * dv, D), lin(m + "o", D, H * dv)
+            w[m + "norm"] = 1.0 + 0.2 * rng.standard_normal(H * dv)
+        else:
+            l, r = mx["left"], mx["right"]
+            H, G, d, dv = int(l["heads"]), int(l["kv_heads"]), int(l["dim"]), int(l["vdim"])
+            p = m + "left."
+            lin(p + "q", H * d, D), lin(p + "k", G * d, D), lin(p + "v", G * dv, D)
+            lin(p + "g", H, D), lin(p + "o", D, H * dv)
+            w[p + "q.norm"] = 1.0 + 0.2 * rng.standard_normal(H * d)
+            w[p + "k.norm"] = 1.0 + 0.2 * rng.standard_normal(G * d)
+            w[p + "sink"] = 1.0 + rng.standard_normal(H)
+            H, d, dv = int(r["heads"]), int(r["dim"]), int(r["vdim"])
+            p = m + "right."
+            lin(p + "q", H * d, D), lin(p + "k", H * d, D), lin(p + "v", H * dv, D)
+            lin(p + "g", H * dv, D), lin(p + "o", D, H * dv)
+            lin(p + "i", H, D, 2.0), lin(p + "f", H, D, 2.0)
+            w[p + "i.b"] = rng.standard_normal(H) - 0.5
+            w[p + "f.b"] = rng.standard_normal(H) + 2.0
+            w[p + "norm"] = 1.0 + 0.2 * rng.standard_normal(H * dv)
+        mlp = L.get("mlp")
+        if not mlp:
+            continue
+        f = a + "mlp."
+        if mlp.get("kind", "dense") == "dense":
+            F = int(mlp["ff"])
+            lin(f + "gate", F, D), lin(f + "up", F, D), lin(f + "down", D, F)
+        else:
+            F, E = int(mlp["expert"]["ff"]), int(mlp["router"]["experts"])
+            lin(f + "router", E, D, 2.0)
+            for e in range(E):
+                lin(f"{f}e{e}.gate", F, D, 1.5), lin(f"{f}e{e}.up", F, D, 1.5)
+                lin(f"{f}e{e}.down", D, F)
+    return {k: bf16_exact(v) for k, v in w.items()}
