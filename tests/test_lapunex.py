@@ -370,6 +370,8 @@ def test_one_layer_models(lay, device, dtype):
 
 @pytest.mark.parametrize("device,dtype", CASES)
 def test_layer_trace_matches_the_oracle(device, dtype):
+    # in bf16 a routing close call moves a whole row and all rows after it: no routing there
+    FULL = globals()["FULL"] if dtype == torch.float32 else without_routing(globals()["FULL"])
     w = O.random_weights(FULL, 2)
     t = toks(14, FULL["vocab"], 4)
     trace = []
@@ -380,8 +382,8 @@ def test_layer_trace_matches_the_oracle(device, dtype):
     assert len(eng.model.layer_trace) == len(trace) == 8          # 1 + 3 * 2 + 1 runs
     for i, (got, want) in enumerate(zip(eng.model.layer_trace, trace)):
         d = np.abs(got.cpu().numpy() - want).max(-1)
-        lim = 1e-3 if dtype == torch.float32 else 0.3
-        assert np.median(d) < lim and (dtype == torch.bfloat16 or d.max() < lim), f"layer {i}"
+        lim = 1e-3 if dtype == torch.float32 else 3e-2 * np.abs(want).max()
+        assert d.max() < lim, f"layer {i}"
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
@@ -535,8 +537,9 @@ def test_first_tokens_and_long_decode(device, dtype, routed):
     pytest.param("cuda", torch.bfloat16, True, marks=pytest.mark.gpu)])
 def test_greedy_generation_through_the_engine(device, dtype, graphs):
     """``LLMEngine.generate``: scheduler, chunked prefill, decode steps (captured graphs and
-    lookahead on the GPU) against greedy decoding with the oracle."""
-    c = copy.deepcopy(FULL)
+    lookahead on the GPU) against greedy decoding with the oracle. In bf16 the model has no
+    routed layers: a routing close call would legitimately change the continuation."""
+    c = copy.deepcopy(FULL) if dtype == torch.float32 else without_routing(FULL)
     w = O.random_weights(c, 12)
     w["head"] = w["head"] * 4.0                          # clear winners
     prompts = [toks(n, c["vocab"], s) for n, s in ((11, 1), (3, 2), (25, 3))]
