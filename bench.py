@@ -203,6 +203,44 @@ def run_design_risutar(a):
                       "results": out}), flush=True)
 
 
+def run_design_lapunex(a):
+    """``--design lapunex``: prefill and decode throughput of the design at layer sizes of a
+    real model (random weights) beside a Mixtral of equal width, depth, heads, expert count,
+    expert width and experts per token, both through ``LLMEngine``. One JSON line."""
+    from dataclasses import replace
+    from distributed_llm_inferencing_amd.models.configs import LayerSpec, get_config, hybrid_config
+    D, Fw, V, Hh, G, hd = a.design_width, a.design_ff, 32000, a.design_width // 128, 8, 128
+    E, top = 8, 2
+    moe = dict(ff_kind="moe", router="group_score", expert_act="clamp_swish", ff=Fw, experts=E,
+               top=top, router_groups=4, router_keep=2, router_scale=1.5, act_limit=7.0)
+
+    def lightning():
+        decays = tuple(1.0 - 2.0 ** (-1.0 - 7.0 * h / max(1, Hh - 1)) for h in range(Hh))
+        return LayerSpec("lightning", heads=Hh, dim=hd, vdim=hd, decays=decays, **moe)
+
+    def parallel():
+        left = LayerSpec("sink_attention", heads=Hh, kv_heads=G, dim=hd, vdim=hd,
+                         scale=hd ** -0.5, rot_dims=64, rot_base=10000.0, window=1 << 30,
+                         rot_scaling=(8.0, 4096.0, 32.0, 1.0))
+        right = LayerSpec("mlstm", heads=Hh // 2, dim=hd, vdim=hd, gate_cap=15.0)
+        return LayerSpec("parallel", heads=Hh, kv_heads=G, dim=hd, vdim=hd, left=left,
+                         right=right, left_scale=0.8, right_scale=0.5, **moe)
+    hyb = hybrid_config("lapunex-bench", D, V, (lightning(), parallel(), lightning(), parallel()),
+                        arch="lapunex", max_position=1 << 15, norm_eps=1e-5, embed_scale=12.0,
+                        streams=3, norm_offset=1.0, loop_entry=False)
+    mix = replace(get_config("mixtral-8x7b"), name="mixtral-bench", hidden_size=D, num_layers=4,
+                  num_heads=Hh, num_kv_heads=G, head_dim=hd, intermediate_size=Fw, vocab_size=V,
+                  num_experts=E, top_k_experts=top, max_position=1 << 15)
+    out = _design_sweep((hyb, mix), a, V)
+    print(json.dumps({"metric": "prefill and decode tokens/s, Lapunex design vs Mixtral of equal "
+                                "size (random weights)", "unit": "tokens/s", "n_gpus": 1,
+                      "dtype": "bf16", "data": "synthetic prompts, random-init weights",
+                      "config": {"width": D, "expert_ff": Fw, "layers": 4, "heads": Hh,
+                                 "kv_heads": G, "head_dim": hd, "memory_heads": Hh // 2,
+                                 "streams": 3, "experts": E, "top": top, "groups": 4, "keep": 2},
+                      "results": out}), flush=True)
+
+
 def run_design(a):
     """``--design buborax``: prefill and decode throughput of the hybrid design at layer sizes
     of a real model (random weights), beside a Llama of equal width, depth (= layer runs),
@@ -427,11 +465,11 @@ def main():
                     help="N>1: pp = layer-sharded pipeline (dense, default), ep = expert "
                          "parallel (MoE), tp = tensor-parallel ablation, dp = independent "
                          "replicas")
-    ap.add_argument("--design", default=None, choices=["buborax", "pulunex", "risutar"],
+    ap.add_argument("--design", default=None, choices=["buborax", "pulunex", "risutar", "lapunex"],
                     help="instead of the headline workload: prefill / decode throughput of "
                          "this design at real layer sizes beside the closest model of equal "
-                         "size (buborax: Llama, pulunex and risutar: Mixtral)")
-    ap.add_argument("--design-models", default="buborax,llama,pulunex,mixtral,risutar",
+                         "size (buborax: Llama, pulunex, risutar and lapunex: Mixtral)")
+    ap.add_argument("--design-models", default="buborax,llama,pulunex,mixtral,risutar,lapunex",
                     help="which of the design and its comparison model to run")
     ap.add_argument("--design-width", type=int, default=4096)
     ap.add_argument("--design-ff", type=int, default=14336)
@@ -445,6 +483,8 @@ def main():
         _heartbeat()
         if a.design == "risutar":
             return run_design_risutar(a)
+        if a.design == "lapunex":
+            return run_design_lapunex(a)
         return run_design_pulunex(a) if a.design == "pulunex" else run_design(a)
 
     from distributed_llm_inferencing_amd import launch

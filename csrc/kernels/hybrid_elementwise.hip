@@ -200,33 +200,44 @@ __device__ __forceinline__ float act_pair(int kind, float g, float u, float limi
 // 3: the exact (erf) GELU of gu[:, c]; 4: gu[:, c] itself (a rounding copy of a column slice);
 // 5: g sigmoid(1.702 g) (u + 1) with g = min(gu[:, c], limit), u = clamp(gu[:, F + c], +-limit).
 // nrows (nullable, device): rows from *nrows on hold no data and are skipped.
-template <typename S>
+// I: the projection's type (fp32, or bf16 bits when a tuned GEMM wrote it).
+template <typename I> __device__ __forceinline__ f32x4 ldin4(const I* p);
+template <> __device__ __forceinline__ f32x4 ldin4<float>(const float* p) {
+  return *reinterpret_cast<const f32x4*>(p);
+}
+template <> __device__ __forceinline__ f32x4 ldin4<u16>(const u16* p) {
+  const uint2 b = *reinterpret_cast<const uint2*>(p);
+  return f32x4{__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u),
+               __uint_as_float(b.y << 16), __uint_as_float(b.y & 0xffff0000u)};
+}
+
+template <typename S, typename I>
 __global__ void __launch_bounds__(256) act_mul_kernel(
-    S* __restrict__ out, int ldo, const float* __restrict__ gu, int ldg, int T, int F, int kind,
+    S* __restrict__ out, int ldo, const I* __restrict__ gu, int ldg, int T, int F, int kind,
     const int* __restrict__ nrows, float limit) {
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid >= (long)T * F) return;
   const int t = (int)(gid / F), c = (int)(gid % F);
   if (nrows != nullptr && t >= *nrows) return;
-  const float* r = gu + (long)t * ldg;
+  const I* r = gu + (long)t * ldg;
   stf(out + (long)t * ldo + c,
-      act_pair(kind, r[c], (kind >= 2 && kind != 5) ? 0.f : r[F + c], limit));
+      act_pair(kind, ldf(r + c), (kind >= 2 && kind != 5) ? 0.f : ldf(r + F + c), limit));
 }
 
 // 4 features a thread (F, ldg multiples of 4, 16-byte aligned rows): 16-byte loads
-template <typename S>
+template <typename S, typename I>
 __global__ void __launch_bounds__(256) act_mul4_kernel(
-    S* __restrict__ out, int ldo, const float* __restrict__ gu, int ldg, int T, int F, int kind,
+    S* __restrict__ out, int ldo, const I* __restrict__ gu, int ldg, int T, int F, int kind,
     const int* __restrict__ nrows, float limit) {
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const int f4 = F >> 2;
   if (gid >= (long)T * f4) return;
   const int t = (int)(gid / f4), c = (int)(gid % f4) * 4;
   if (nrows != nullptr && t >= *nrows) return;
-  const float* r = gu + (long)t * ldg;
-  const f32x4 g = *reinterpret_cast<const f32x4*>(r + c);
+  const I* r = gu + (long)t * ldg;
+  const f32x4 g = ldin4(r + c);
   f32x4 u = f32x4{0.f, 0.f, 0.f, 0.f};
-  if (kind < 2 || kind == 5) u = *reinterpret_cast<const f32x4*>(r + F + c);
+  if (kind < 2 || kind == 5) u = ldin4(r + F + c);
 #pragma unroll
   for (int i = 0; i < 4; ++i)
     stf(out + (long)t * ldo + c + i, act_pair(kind, g[i], u[i], limit));
@@ -459,20 +470,27 @@ extern "C" int dli_token_shift(const float* h, const void* mu, float* state, con
   DLI_RETURN_LAUNCH();
 }
 
-extern "C" int dli_act_mul(void* out, int ldo, const float* gu, int ldg, int T, int F, int kind,
-                           const int* nrows, float limit, int dt, hipStream_t st) {
+// in_dt: type of the projection gu (1 fp32; 0 bf16, with bf16 output only)
+extern "C" int dli_act_mul(void* out, int ldo, const void* gu, int ldg, int T, int F, int kind,
+                           const int* nrows, float limit, int in_dt, int dt, hipStream_t st) {
   if (T <= 0) return 0;
-  if (kind < 0 || kind > 5) return (int)hipErrorInvalidValue;
-  if (F % 4 == 0 && ldg % 4 == 0 && (uintptr_t)gu % 16 == 0) {
-    const int nb4 = (int)(((long)T * (F / 4) + 255) / 256);
-    DT_SWITCH(dt,
-              (act_mul4_kernel<u16><<<nb4, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F, kind, nrows, limit)),
-              (act_mul4_kernel<float><<<nb4, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F, kind, nrows, limit)));
+  if (kind < 0 || kind > 5 || in_dt < 0 || in_dt > 1 || (in_dt == 0 && dt != 0))
+    return (int)hipErrorInvalidValue;
+  const bool v4 = F % 4 == 0 && ldg % 4 == 0 && (uintptr_t)gu % 16 == 0;
+  const int nb = (int)(((long)T * (v4 ? F / 4 : F) + 255) / 256);
+  if (in_dt == 0) {
+    if (v4) act_mul4_kernel<u16, u16><<<nb, 256, 0, st>>>((u16*)out, ldo, (const u16*)gu, ldg, T, F, kind, nrows, limit);
+    else act_mul_kernel<u16, u16><<<nb, 256, 0, st>>>((u16*)out, ldo, (const u16*)gu, ldg, T, F, kind, nrows, limit);
     DLI_RETURN_LAUNCH();
   }
-  const int nb = (int)(((long)T * F + 255) / 256);
-  DT_SWITCH(dt, (act_mul_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, ldo, gu, ldg, T, F, kind, nrows, limit)),
-            (act_mul_kernel<float><<<nb, 256, 0, st>>>((float*)out, ldo, gu, ldg, T, F, kind, nrows, limit)));
+  const float* gf = (const float*)gu;
+  if (v4)
+    DT_SWITCH(dt,
+              (act_mul4_kernel<u16, float><<<nb, 256, 0, st>>>((u16*)out, ldo, gf, ldg, T, F, kind, nrows, limit)),
+              (act_mul4_kernel<float, float><<<nb, 256, 0, st>>>((float*)out, ldo, gf, ldg, T, F, kind, nrows, limit)));
+  else
+    DT_SWITCH(dt, (act_mul_kernel<u16, float><<<nb, 256, 0, st>>>((u16*)out, ldo, gf, ldg, T, F, kind, nrows, limit)),
+              (act_mul_kernel<float, float><<<nb, 256, 0, st>>>((float*)out, ldo, gf, ldg, T, F, kind, nrows, limit)));
   DLI_RETURN_LAUNCH();
 }
 

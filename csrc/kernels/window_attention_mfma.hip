@@ -71,6 +71,11 @@ struct MfmaArgs {
   // > 0: the cache rows of the whole window (slot_cap ints) are looked up once at kernel start
   // instead of per key tile (one global round trip and one barrier less per tile)
   int slot_cap;
+  // sink != null (forms without head mixing): exp(sink[h]) joins head h's softmax denominator,
+  // a key without a value counted once: the running (max, sum) of the first key split start
+  // from (sink, 1) instead of (-inf, 0). head_gate: the gate row holds one number per head.
+  // out_scale multiplies the output.
+  const float* sink; int head_gate; float out_scale;
   float* stats_ws;   // [S][q tiles][nsplit][H][TQ][2]
   float* o_ws;       // [nsplit][T][H*dv]
   long o_ws_stride;  // T * H * dv
@@ -158,6 +163,15 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
     l_run[hh] = 0.f;
 #pragma unroll
     for (int b = 0; b < MAXDVB; ++b) oacc[hh][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  if (a.sink != nullptr && (a.nsplit <= 1 || split == 0)) {
+#pragma unroll
+    for (int hh = 0; hh < MAXHW; ++hh) {
+      const int h = wide ? hbase + wave : wave + hh * NW;
+      if (h >= H || (wide && hh)) continue;
+      m_run[hh] = a.sink[h] * LOG2E;              // scores live in the log2 domain
+      l_run[hh] = 1.f;
+    }
   }
   const int nf = dq >> 5;                         // 32-wide K-steps of the score product
   const float scale2 = a.scale * LOG2E;
@@ -541,7 +555,8 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
       for (int r = 0; r < 4; ++r) {
         o[r] = oacc[hh][b][r] * onorm;
         if (a.gate != nullptr)
-          o[r] *= 1.f / (1.f + expf(-a.gate[(long)(t0 + fr) * a.ldg + col + r]));
+          o[r] *= 1.f / (1.f + expf(-a.gate[(long)(t0 + fr) * a.ldg + (a.head_gate ? h : col + r)]));
+        o[r] *= a.out_scale;
       }
       uint2 pk;
       pk.x = pack2bf(o[0], o[1]);
@@ -555,7 +570,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
 __global__ void __launch_bounds__(256) split_reduce_kernel(
     u16* __restrict__ out, int ldo, const float* __restrict__ o_ws, long stride, int nsplit,
     const float* __restrict__ gate, int ldg, int T, int width, const float* __restrict__ stats,
-    int H, int dv) {
+    int H, int dv, int head_gate, float out_scale) {
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const int w4 = width >> 2;
   if (gid >= (long)T * w4) return;
@@ -580,8 +595,10 @@ __global__ void __launch_bounds__(256) split_reduce_kernel(
   }
   if (gate != nullptr) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) acc[r] *= 1.f / (1.f + expf(-gate[(long)t * ldg + c + r]));
+    for (int r = 0; r < 4; ++r)
+      acc[r] *= 1.f / (1.f + expf(-gate[(long)t * ldg + (head_gate ? c / dv : c + r)]));
   }
+  acc *= out_scale;
   uint2 pk;
   pk.x = pack2bf(acc[0], acc[1]);
   pk.y = pack2bf(acc[2], acc[3]);
@@ -634,7 +651,9 @@ extern "C" int dli_window_attention_mfma(
     hipStream_t st) {
   if (num_seqs <= 0 || max_seqlen <= 0) return 0;
   if (chunk < 0 || Gk < 1) return (int)hipErrorInvalidValue;
-  if (sink != nullptr || head_gate || out_scale != 1.f) return (int)hipErrorNotSupported;
+  // the sink rides on the one-pass forms' running (max, sum); with head mixing it has no place
+  if (sink != nullptr && (talk != nullptr || rowhead)) return (int)hipErrorNotSupported;
+  if (head_gate && dv % 4) return (int)hipErrorNotSupported;
   // keys a query tile can see: bounds the slot table and the key splits
   const int weff = chunk > 0 && chunk < window ? chunk : window;
   int rowmul = 1, vrows = 0;
@@ -706,7 +725,7 @@ extern "C" int dli_window_attention_mfma(
   MfmaArgs a{(const u16*)q, ldq, (const u16*)k, k_stride, (const u16*)v, v_stride, (u16*)out,
              ldo, gate, ldg, slopes, talk, cu, positions, block_tables, bt_stride, block_size,
              H, G, dq, dv, window, scale, Gk, chunk, Hp, CG, 0, 1, ndvs, wide ? 1 : 0, nhs, rowmul,
-             vrows, cgv, slot_cap, nullptr, nullptr, 0};
+             vrows, cgv, slot_cap, sink, head_gate, out_scale, nullptr, nullptr, 0};
   if (nsplit == 1) {
     dim3 grid(qtiles, num_seqs, ndvs * nhs);
     WA_LAUNCH(grid);
@@ -726,7 +745,8 @@ extern "C" int dli_window_attention_mfma(
     a.mode = 3;
     WA_LAUNCH(dim3(qtiles, num_seqs, ndvs * nhs * nsplit));
     split_reduce_kernel<<<(int)((quads + 255) / 256), 256, 0, st>>>(
-        (u16*)out, ldo, a.o_ws, a.o_ws_stride, nsplit, gate, ldg, T, H * dv, a.stats_ws, H, dv);
+        (u16*)out, ldo, a.o_ws, a.o_ws_stride, nsplit, gate, ldg, T, H * dv, a.stats_ws, H, dv,
+        head_gate, out_scale);
     DLI_RETURN_LAUNCH();
   }
   a.mode = 1;
@@ -736,6 +756,7 @@ extern "C" int dli_window_attention_mfma(
   a.ndvs = ndvs;
   WA_LAUNCH(dim3(qtiles, num_seqs, ndvs * nhs * nsplit));
   split_reduce_kernel<<<(int)((quads + 255) / 256), 256, 0, st>>>(
-      (u16*)out, ldo, a.o_ws, a.o_ws_stride, nsplit, gate, ldg, T, H * dv, nullptr, H, dv);
+      (u16*)out, ldo, a.o_ws, a.o_ws_stride, nsplit, gate, ldg, T, H * dv, nullptr, H, dv,
+      head_gate, out_scale);
   DLI_RETURN_LAUNCH();
 }

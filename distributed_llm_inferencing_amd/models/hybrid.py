@@ -277,6 +277,7 @@ class HybridLM(TransformerLM):
         for spec, lp in zip(self.cfg.layer_specs, self.layers):
             if spec.ff_kind == "moe" and "ff_tuned" in lp:
                 w1, epi = ((lp["w_up"], "gelu_erf") if spec.expert_act == "gelu_erf"
+                           else (lp["w_gu"], "none") if spec.expert_act == "clamp_swish"
                            else (lp["w_gu"], "silu_mul"))
                 key = (tuple(w1.shape), spec.top, epi)
                 if key not in seen:

@@ -247,7 +247,6 @@ def prepare_feed_forward(spec: LayerSpec, params: dict, pre: str) -> None:
     w = params.get(pre + "w_down")
     if (not spec.ff or w is None or pre + "ff_tuned" in params or w.dtype != torch.bfloat16
             or not w.is_cuda or spec.ff_kind not in ("gelu", "moe", "gated_silu")
-            or spec.expert_act == "clamp_swish"
             or w.shape[-2] % 64 or spec.ff % 64 or spec.shared_ff % 64):
         return
     if spec.ff_kind == "gelu":
@@ -255,6 +254,8 @@ def prepare_feed_forward(spec: LayerSpec, params: dict, pre: str) -> None:
     elif spec.ff_kind == "gated_silu":
         gu = params[pre + "w_gu"]
         params[pre + "w_gu"] = interleave_gate_up(gu[:spec.ff], gu[spec.ff:]).contiguous()
+    elif spec.ff_kind == "moe" and spec.expert_act == "clamp_swish":
+        pass                                         # the plain [gate | up] weight serves
     elif spec.expert_act == "silu_mul":
         gu = params[pre + "w_gu"]
         for e in range(gu.shape[0]):                 # expert by expert: no second full copy
@@ -296,8 +297,13 @@ def moe_ff(spec: LayerSpec, lp: dict, h):
     if spec.router == "group_score":
         tw, ti, _ = H.score_router(h, lp["router"], None, spec.top, 0, spec.router_groups,
                                    spec.router_keep, spec.router_scale)
-        return H.moe_experts_f32(h, lp["w_gu"], lp["w_down"], tw, ti, None, act="clamp_swish",
-                                 limit=spec.act_limit)
+        if "ff_tuned" not in lp:
+            return H.moe_experts_f32(h, lp["w_gu"], lp["w_down"], tw, ti, None,
+                                     act="clamp_swish", limit=spec.act_limit)
+        from .. import ops
+        routed = ops.moe_mlp(h, lp["w_gu"], lp["w_down"], tw, ti, 0, act="clamp_swish",
+                             limit=spec.act_limit)
+        return H.moe_finish(routed, tw, ti, h, lp["w_gu"].shape[0])
     if spec.router == "logit_topk":
         tw, ti = H.logit_router(h, lp["router"], lp["router_b"], spec.top)
         if "ff_tuned" not in lp:

@@ -692,11 +692,14 @@ def moe_router(h, w_router, k: int):
 
 def moe_mlp(x, w_gu, w_down, topk_w, topk_ids, expert_offset: int = 0,
             plan_rows: Optional[int] = None, defer_combine: bool = False,
-            act: str = "silu_mul"):
+            act: str = "silu_mul", limit: float = 0.0):
     """Experts [expert_offset, expert_offset+E_local) of one MoE layer; returns the weighted
     sum over the token's selected local experts (zeros for tokens routed elsewhere).
     ``act``: ``silu_mul`` (gated experts, ``w_gu`` = the interleaved gate/up weight) or
-    ``gelu_erf`` (ungated experts down(gelu(up x)), ``w_gu`` = the up weight [E, F, D]).
+    ``gelu_erf`` (ungated experts down(gelu(up x)), ``w_gu`` = the up weight [E, F, D]) or
+    ``clamp_swish`` (gated experts with the clamped activation of ``ops.hybrid.act_mul``, its
+    clamp ``limit`` a per-model constant: ``w_gu`` = the plain [gate | up] weight [E, 2F, D];
+    the gate/up GEMM writes bf16 and one elementwise kernel applies the activation).
     ``plan_rows``: the routed rows these experts typically receive, when ``x`` is a region
     sized for the worst case (the expert-parallel receive region: every peer's bucket at
     min(k, E/N) rows per token). The grouped-GEMM plan is looked up for it — the autotuned
@@ -710,7 +713,8 @@ def moe_mlp(x, w_gu, w_down, topk_w, topk_ids, expert_offset: int = 0,
     k = topk_ids.shape[1]
     E_local, F2, _ = w_gu.shape
     gated = act == "silu_mul"
-    Fa = F2 // 2 if gated else F2              # width of the activation
+    clamped = act == "clamp_swish"
+    Fa = F2 // 2 if gated or clamped else F2   # width of the activation
     n = T * k
     dev = x.device
     offsets = torch.empty(E_local + 1, dtype=torch.int32, device=dev)
@@ -718,8 +722,14 @@ def moe_mlp(x, w_gu, w_down, topk_w, topk_ids, expert_offset: int = 0,
     src = torch.empty(max(n, 1), dtype=torch.int32, device=dev)
     _native_call("dli_moe_align", _p(offsets), _p(pos), _p(src), _p(topk_ids), n, k,
                  expert_offset, E_local, _st())
-    epi_up = act
-    act = torch.empty(max(n, 1), Fa, dtype=x.dtype, device=dev)
+    epi_up = "none" if clamped else act
+    act = torch.empty(max(n, 1), F2 if clamped else Fa, dtype=x.dtype, device=dev)
+
+    def finish_act(a):
+        if not clamped:
+            return a
+        from . import hybrid as _H
+        return _H.act_mul(a, Fa, x.dtype, "clamp_swish", rows=offsets[E_local:], limit=limit)
     if n >= _MOE_PREFILL_ROWS * E_local and not torch.cuda.is_current_stream_capturing():
         # prefill-sized expert GEMMs (thousands of rows per expert) are compute-bound: a
         # grouped 256x256 kernel (G.MOE_PREFILL_TILE: the two-barrier 4-wave tile, grid.z =
@@ -738,6 +748,7 @@ def moe_mlp(x, w_gu, w_down, topk_w, topk_ids, expert_offset: int = 0,
             p_up = p8 if G.tile_ok(p8.tile, epi_up) else G.GemmPlan("dli", 22, 1)
             _gemm_native(xp, w_gu, epi_up, out=act, groups=E_local, group_off=offsets,
                          rows_per_group=rows_max, plan=p_up)
+            act = finish_act(act)
             _gemm_native(act, w_down, "none", out=y, groups=E_local, group_off=offsets,
                          rows_per_group=rows_max, plan=p8)
         out = torch.empty_like(x)
@@ -758,6 +769,7 @@ def moe_mlp(x, w_gu, w_down, topk_w, topk_ids, expert_offset: int = 0,
                      _st())
         _gemm_native(xp, w_gu, epi_up, out=act, groups=E_local, group_off=offsets,
                      rows_per_group=n, plan=p_gu)
+    act = finish_act(act)
     p_dn = G.grouped_plan(rows, D, Fa, "none", E_local)
     if moe_slab_plan(p_dn):
         if defer_combine:

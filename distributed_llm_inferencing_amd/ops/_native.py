@@ -76,7 +76,7 @@ _SIGS = {
     "dli_embedding_f32": [P, P, P, P, I, I, I, F, P, P, I, I, P],
     "dli_resadd_groupnorm": [P, P, I, P, F, F, P, P, I, I, I, I, F, P, F, I, F, I, P],
     "dli_token_shift": [P, P, P, P, P, P, P, I, I, I, I, P],
-    "dli_act_mul": [P, I, P, I, I, I, I, P, F, I, P],
+    "dli_act_mul": [P, I, P, I, I, I, I, P, F, I, I, P],
     "dli_talk_prepare": [P, I, P, P, F, I, I, I, I, I, P, P, P, P, I, P],
     "dli_score_router": [P, P, P, P, I, P, P, I, I, I, I, I, I, I, F, I, P],
     "dli_gemm_any_grouped": [P, L, P, L, L, P, L, I, I, I, I, I, P, P, P],

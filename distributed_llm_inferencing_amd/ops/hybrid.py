@@ -185,6 +185,7 @@ def act_mul(gu: torch.Tensor, F_: int, dtype, kind: str = "gelu_mul",
     act(gu[:, :F]) * gu[:, F:2F]; ``gelu`` = gelu_tanh(gu[:, :F]); ``gelu_erf`` = the exact GELU
     of gu[:, :F]; ``copy`` = gu[:, :F] rounded to the storage dtype; ``clamp_swish`` = g
     sigmoid(1.702 g) (u + 1) with g = min(gu[:, :F], limit), u = clamp(gu[:, F:2F], +-limit).
+    ``gu`` may also be a bf16 projection (a tuned GEMM's output) when ``dtype`` is bf16.
     ``rows`` (device int32
     scalar): only that many leading rows hold data (routed rows of a mixture)."""
     if not gu.is_cuda:
@@ -192,7 +193,7 @@ def act_mul(gu: torch.Tensor, F_: int, dtype, kind: str = "gelu_mul",
     T = gu.shape[0]
     out = torch.empty(T, F_, dtype=dtype, device=gu.device)
     _call("dli_act_mul", _p(out), F_, _p(gu), gu.stride(0), T, F_, _ACT_KINDS[kind], _p(rows),
-          float(limit), _dt(dtype), _st())
+          float(limit), _dt(gu.dtype), _dt(dtype), _st())
     return out
 
 

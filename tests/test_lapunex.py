@@ -597,3 +597,29 @@ def test_registry_model_random_init_generates():
     outs = eng.generate([[1, 2, 3], [4, 5, 6, 7, 8]], SamplingParams(max_new_tokens=4, do_sample=False,
                                                                     ignore_eos=True))
     assert all(len(o.output_ids) == 4 for o in outs)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("width,lay,n", [
+    (128, lightning(heads=2, dim=16, vdim=32, mlp=moe(ff=64, experts=4, top=2, groups=(2, 1))), 70),
+    (64, parallel(l=left(heads=4, kv_heads=2, dim=32, vdim=16, rot_=rot(8)),
+                  r=right(heads=2, dim=16, vdim=16), mlp=moe(ff=128, experts=3, top=1, groups=None)), 33),
+    (128, lightning(heads=1, dim=32, vdim=64, mlp=dense(192)), 41),
+    (192, parallel(l=left(heads=8, kv_heads=2, dim=64, vdim=32, scale=0.12, rot_=rot(16, 1000.0)),
+                   r=right(heads=2, dim=64, vdim=64),
+                   mlp=moe(ff=64, experts=8, top=3, groups=(4, 3))), 300)],
+    ids=["lightning_moe", "parallel_moe_top1", "dense", "matrix_core_attention"])
+def test_tuned_layouts_and_matrix_core_attention(width, lay, n):
+    """Sizes the tuned GEMM tiles and the matrix-core attention take: the dense feed-forward's
+    activation runs as a GEMM epilogue, the experts as grouped GEMMs, the attention (sink,
+    head gates, output scale) on the MFMA kernel, also split over keys for single tokens at a
+    long context; whole prompts, portions and single tokens."""
+    c = config([lay, lay], width=width, vocab=96)
+    w = O.random_weights(c, width + n)
+    t = toks(n, 96, n)
+    want = ref(t, c, w)
+    eng = engine(c, w, "cuda", torch.bfloat16, max_tokens=640)
+    assert "ff_tuned" in eng.model.layers[0]
+    close(replay(eng, t, [n]), want, torch.bfloat16, "whole")
+    close(replay(eng, t, [n - 9, 2, 1, 1, 5]), want, torch.bfloat16, "portions")
+    close(replay(eng, t, [n - 20] + [1] * 20), want, torch.bfloat16, "decoded")
