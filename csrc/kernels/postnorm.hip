@@ -205,11 +205,17 @@ __global__ void __launch_bounds__(256) side_gate_kernel(
 template <typename S>
 __global__ void __launch_bounds__(256) rmsnorm_cols_kernel(
     S* __restrict__ out, const float* __restrict__ src, int lds, const S* __restrict__ w, int T,
-    int n, float eps, bool vec4, const float* __restrict__ gate, int ldg) {
+    int n, float eps, bool vec4, const float* __restrict__ gate, int ldg, int groups, int ldo,
+    float out_scale) {
+  // a row = one of `groups` parts (n wide each, normed by itself) of a token's row
   const int lane = threadIdx.x & 63;
-  const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (t >= T) return;
-  const float* r = src + (long)t * lds;
+  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= T * groups) return;
+  const int t = row / groups, go = (row % groups) * n;
+  const float* r = src + (long)t * lds + go;
+  w += go;
+  out += (long)t * ldo + go;
+  if (gate != nullptr) gate += (long)t * ldg + go;
   float s = 0.f;
   if (vec4) {                                   // 16-byte loads, 4 columns a lane
     for (int c = lane * 4; c < n; c += 256) {
@@ -221,11 +227,11 @@ __global__ void __launch_bounds__(256) rmsnorm_cols_kernel(
     for (int c = lane * 4; c < n; c += 256) {
       f32x4 v = *reinterpret_cast<const f32x4*>(r + c) * rs * ld4(w + c);
       if (gate != nullptr) {
-        const f32x4 g = *reinterpret_cast<const f32x4*>(gate + (long)t * ldg + c);
+        const f32x4 g = *reinterpret_cast<const f32x4*>(gate + c);
 #pragma unroll
         for (int u = 0; u < 4; ++u) v[u] *= 1.f / (1.f + expf(-g[u]));
       }
-      st4(out + (long)t * n + c, v);
+      st4(out + c, v * out_scale);
     }
     return;
   }
@@ -234,8 +240,8 @@ __global__ void __launch_bounds__(256) rmsnorm_cols_kernel(
   const float rs = 1.f / sqrtf(s / (float)n + eps);
   for (int c = lane; c < n; c += 64) {
     float v = r[c] * rs * ldf(w + c);
-    if (gate != nullptr) v *= 1.f / (1.f + expf(-gate[(long)t * ldg + c]));
-    stf(out + (long)t * n + c, v);
+    if (gate != nullptr) v *= 1.f / (1.f + expf(-gate[c]));
+    stf(out + c, v * out_scale);
   }
 }
 
@@ -472,18 +478,20 @@ extern "C" int dli_side_gate(void* out, const float* gate, int ldg, const int* i
 }
 
 extern "C" int dli_rmsnorm_cols(void* out, const float* src, int lds, const void* w, int T, int n,
-                                float eps, const float* gate, int ldg, int dt, hipStream_t st) {
+                                float eps, const float* gate, int ldg, int groups, int ldo,
+                                float out_scale, int dt, hipStream_t st) {
   if (T <= 0) return 0;
-  if (n < 1) return (int)hipErrorInvalidValue;
-  const int nb = (T + 3) / 4;
-  const bool vec4 = n % 4 == 0 && lds % 4 == 0 && ldg % 4 == 0 &&
+  if (n < 1 || groups < 1) return (int)hipErrorInvalidValue;
+  const int nb = (int)(((long)T * groups + 3) / 4);
+  const bool vec4 = n % 4 == 0 && lds % 4 == 0 && ldg % 4 == 0 && ldo % 4 == 0 &&
                     (((uintptr_t)out | (uintptr_t)src | (uintptr_t)w | (uintptr_t)gate) & 15) == 0;
   DT_SWITCH(dt,
             (rmsnorm_cols_kernel<u16><<<nb, 256, 0, st>>>((u16*)out, src, lds, (const u16*)w, T,
-                                                          n, eps, vec4, gate, ldg)),
+                                                          n, eps, vec4, gate, ldg, groups, ldo,
+                                                          out_scale)),
             (rmsnorm_cols_kernel<float><<<nb, 256, 0, st>>>((float*)out, src, lds,
                                                             (const float*)w, T, n, eps, vec4,
-                                                            gate, ldg)));
+                                                            gate, ldg, groups, ldo, out_scale)));
   DLI_RETURN_LAUNCH();
 }
 

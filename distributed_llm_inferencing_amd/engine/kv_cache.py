@@ -99,10 +99,10 @@ class HybridCache:
                             nothing)
 
     * ``lightning``:        (state [state_slots, H, d, dv] fp32,)
-    * ``parallel``:         (k [slots, G*d], v [slots, G*dv], state [state_slots, Hr, dr,
-                            dvr + 1] fp32, m [state_slots, Hr] fp32): the attention side's
-                            normed, rotated keys and values; the memory side's matrix with its
-                            normaliser vector as one more column, and its running maximum
+    * ``parallel``:         (k [slots, G*d], v [slots, G*dv], state [state_slots, Hr, dr, dvr]
+                            fp32, nm [state_slots, Hr, dr + 1] fp32): the attention side's
+                            normed, rotated keys and values; the memory side's matrix, and its
+                            normaliser vector followed by its running maximum
 
     ``shift_states[run]`` is [state_slots, D] fp32 for a layer with token shift (the previous
     token's mixer input), else None. ``prev_token`` is int32 [state_slots] for a design whose
@@ -152,9 +152,10 @@ class HybridCache:
                 l, r = s.left, s.right
                 e = (torch.zeros(rows, l.kv_heads * l.dim, dtype=dtype, device=device),
                      torch.zeros(rows, l.kv_heads * l.vdim, dtype=dtype, device=device),
-                     torch.zeros(state_slots, r.heads, r.dim, r.vdim + 1, dtype=torch.float32,
+                     torch.zeros(state_slots, r.heads, r.dim, r.vdim, dtype=torch.float32,
                                  device=device),
-                     torch.zeros(state_slots, r.heads, dtype=torch.float32, device=device))
+                     torch.zeros(state_slots, r.heads, r.dim + 1, dtype=torch.float32,
+                                 device=device))
             else:
                 e = (torch.zeros(state_slots, s.heads, s.dim, s.vdim, dtype=torch.float32,
                                  device=device),)

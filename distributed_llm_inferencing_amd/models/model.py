@@ -64,6 +64,8 @@ class TransformerLM:
                                       le == cfg.num_layers, None)
         params = W.random_init(shapes, device, dtype, seed,
                                 norm_value=1.0 - cfg.norm_offset)
+        if cfg.is_hybrid:
+            W.calm_random_mixers(cfg, params)
         if expert_range is not None:
             params = {k: W.slice_experts(k, v, expert_range) for k, v in params.items()}
         return cls(cfg, params, layer_start, le, device, expert_range)

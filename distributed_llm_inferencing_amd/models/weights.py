@@ -291,6 +291,17 @@ def _hybrid_init(name: str, shape: tuple, dev, dtype, seed: int) -> torch.Tensor
     return (torch.randn(shape, generator=g) / shape[-1] ** 0.5).to(dev, dtype)
 
 
+def calm_random_mixers(cfg: ModelConfig, params: Dict[str, torch.Tensor]) -> None:
+    """Random-init only. A fixed-decay linear attention reads SiLU-activated (mostly positive)
+    queries, keys and values, so at random init its output has a large component shared by
+    all tokens, which makes a random router send every token to the same experts (a trained
+    model's routing is spread). Its output projection therefore starts small."""
+    for i, s in enumerate(cfg.layer_specs):
+        k = f"layers.{i}.wo"
+        if s.kind == "lightning" and k in params:
+            params[k].mul_(0.1)
+
+
 def slice_experts(name: str, t: torch.Tensor, expert_range: Optional[tuple]) -> torch.Tensor:
     if expert_range is None or not (name.endswith(".w_gu") or name.endswith(".w_down")):
         return t

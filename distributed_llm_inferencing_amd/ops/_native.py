@@ -97,7 +97,7 @@ _SIGS = {
     "dli_postnorm": [P, P, I, F, P, P, P, I, I, F, P, I, P],
     "dli_add_rmsnormed": [P, P, I, P, P, I, I, F, I, P],
     "dli_side_gate": [P, P, I, P, P, I, I, I, I, I, I, P],
-    "dli_rmsnorm_cols": [P, P, I, P, I, I, F, P, I, I, P],
+    "dli_rmsnorm_cols": [P, P, I, P, I, I, F, P, I, I, I, F, I, P],
     "dli_latent_prepare": [P, I, P, I, P, F, I, I, I, I, I, I, P, P, P, P, P, P, I, I, P],
     "dli_head_gate": [P, P, P, I, I, I, I, I, P],
     "dli_logit_router": [P, P, P, I, P, P, I, I, I, I, I, P],
@@ -105,7 +105,7 @@ _SIGS = {
     "dli_hyper_mix": [P, P, I, P, P, P, P, I, I, I, F, F, I, P],
     "dli_sink_prepare": [P, I, P, P, F, I, I, I, I, I, I, P, F, P, P, P, P, P, I, P],
     "dli_scalar_recurrence": [P, I, I, P, P, F, P, F, P, P, P, P, P, P, I, F, I, I, I, I, I,
-                              I, P],
+                              I, P, I, P],
 }
 
 

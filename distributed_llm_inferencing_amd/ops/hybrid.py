@@ -476,16 +476,28 @@ def side_gate(gate, ids, table, col0: int) -> torch.Tensor:
     return out
 
 
-def rmsnorm_cols(src, w, eps: float, gate=None) -> torch.Tensor:
+def rmsnorm_cols(src, w, eps: float, gate=None, groups: int = 1, out=None,
+                 out_scale: float = 1.0) -> torch.Tensor:
     """RMS norm times w of the rows of an fp32 matrix that may be a column slice of a wider
-    one, times sigmoid(gate) (fp32, same shape, may be a column slice) when given; storage
-    dtype out."""
+    one, times sigmoid(gate) (fp32, same shape, may be a column slice) when given, times
+    ``out_scale``; storage dtype out. With ``groups`` > 1 each row is that many equal parts,
+    each normed by itself (heads). ``out`` may be a column slice of a wider buffer."""
     if not src.is_cuda:
-        return R.rmsnorm_cols(src, w, eps, w.dtype, gate)
+        T, n = src.shape
+        o = R.rmsnorm_cols(src.reshape(T * groups, n // groups),
+                           w.reshape(groups, n // groups).repeat(T, 1), eps, torch.float32,
+                           gate.reshape(T * groups, n // groups) if gate is not None else None)
+        o = (o.reshape(T, n) * out_scale).to(w.dtype)
+        if out is not None:
+            out.copy_(o)
+            return out
+        return o
     T, n = src.shape
-    out = torch.empty(T, n, dtype=w.dtype, device=src.device)
-    _call("dli_rmsnorm_cols", _p(out), _p(src), src.stride(0), _p(w), T, n, float(eps),
-          _p(gate), gate.stride(0) if gate is not None else 0, _dt(w.dtype), _st())
+    if out is None:
+        out = torch.empty(T, n, dtype=w.dtype, device=src.device)
+    _call("dli_rmsnorm_cols", _p(out), _p(src), src.stride(0), _p(w), T, n // groups,
+          float(eps), _p(gate), gate.stride(0) if gate is not None else 0, int(groups),
+          out.stride(0), float(out_scale), _dt(w.dtype), _st())
     return out
 
 
@@ -629,21 +641,37 @@ def lightning(proj, decays, state, slots, cu_seqlens, max_seqlen, positions, H, 
     out = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
     _call("dli_scalar_recurrence", _p(proj), proj.stride(0), 0, _p(decays), None, 0.0, None, 0.0,
           _p(state), None, _p(slots), _p(cu_seqlens), _p(positions), _p(out), out.stride(0), 1.0,
-          S, int(max_seqlen), H, d, dv, 1, _st())
+          S, int(max_seqlen), H, d, dv, _column_block(S, H, dv, max_seqlen), None, 1, _st())
     return out
+
+
+def _column_block(S: int, H: int, dv: int, max_seqlen: int) -> int:
+    """State columns per workgroup of a recurrence over a step's portions: few (head,
+    sequence) pairs with long portions leave most of the chip idle, so the columns are dealt
+    to several workgroups (0: one workgroup holds all of them)."""
+    return 64 if (S * H < 256 and max_seqlen >= 64 and dv >= 128) else 0
 
 
 def mlstm(proj, if_b, cap: float, norm_w, eps: float, state, mstate, slots, cu_seqlens,
           max_seqlen, positions, H, d, dv, out, out_scale: float = 1.0):
     """Matrix memory with exponential gating over per-sequence state slots
     (``reference.mlstm``); the normed, gated, scaled read-out is written to ``out`` [T, H*dv]
-    (storage dtype; may be a column slice of a wider buffer)."""
+    (storage dtype; may be a column slice of a wider buffer). ``state`` fp32 [slots, H, d, dv];
+    ``mstate`` fp32 [slots, H, d + 1] holds the normaliser vector and the running maximum."""
     if not proj.is_cuda:
         return R.mlstm(proj, if_b, cap, norm_w, eps, state, mstate, slots, cu_seqlens, positions,
                        H, d, dv, out, out_scale)
     S = cu_seqlens.shape[0] - 1
+    cw = _column_block(S, H, dv, max_seqlen)
+    # with column blocks no workgroup sees a whole head: the read-outs leave in fp32 and the
+    # per-head norm, gate and scale run as a row kernel
+    raw = torch.empty(proj.shape[0], H * dv, dtype=torch.float32, device=proj.device) if cw else None
     _call("dli_scalar_recurrence", _p(proj), proj.stride(0), 1, None, _p(if_b), float(cap),
           _p(norm_w), float(eps), _p(state), _p(mstate), _p(slots), _p(cu_seqlens),
           _p(positions), _p(out), out.stride(0), float(out_scale), S, int(max_seqlen), H, d, dv,
-          _dt(norm_w.dtype), _st())
+          cw, _p(raw), _dt(norm_w.dtype), _st())
+    if cw:
+        g0 = 2 * H * d + H * dv
+        rmsnorm_cols(raw, norm_w, eps, gate=proj[:, g0:g0 + H * dv], groups=H, out=out,
+                     out_scale=out_scale)
     return out

@@ -901,8 +901,8 @@ def mlstm(proj, if_b, cap, norm_w, eps, state, mstate, slots, cu_seqlens, positi
         m' = max(f + m, i);  S = e^(f + m - m') S + e^(i - m') k v^T;  n likewise with k alone;
         o = S^T q d^(-1/2) / (max(|n . q d^(-1/2)|, e^(-m')) + 1e-6)
     o is RMS-normed per head, times norm_w [H*dv], sigmoid(gate) and out_scale, and written to
-    ``out`` [T, H*dv]. state fp32 [slots, H, d, dv + 1] holds S and, as its last column, n;
-    mstate fp32 [slots, H] holds m."""
+    ``out`` [T, H*dv]. state fp32 [slots, H, d, dv] holds S; mstate fp32 [slots, H, d + 1] holds
+    n and, last, m."""
     T = proj.shape[0]
     cu, sl = cu_seqlens.tolist(), slots.tolist()
     nw = norm_w.float().reshape(H, dv)
@@ -914,8 +914,8 @@ def mlstm(proj, if_b, cap, norm_w, eps, state, mstate, slots, cu_seqlens, positi
         if sl[s] < 0:
             out[t0:t1] = 0
             continue
-        S = state[sl[s]].clone()
-        m = mstate[sl[s]].clone()
+        S = torch.cat([state[sl[s]], mstate[sl[s]][:, :d, None]], 2)      # [H, d, dv + 1]
+        m = mstate[sl[s]][:, d].clone()
         if int(positions[t0]) == 0:
             S.zero_()
             m.zero_()
@@ -939,8 +939,8 @@ def mlstm(proj, if_b, cap, norm_w, eps, state, mstate, slots, cu_seqlens, positi
             o = r[:, :dv] / (torch.maximum(r[:, dv:].abs(), torch.exp(-m)[:, None]) + 1e-6)
             o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * nw
             out[t0 + t] = (o * torch.sigmoid(gv[t]) * out_scale).reshape(H * dv).to(out.dtype)
-        state[sl[s]] = S
-        mstate[sl[s]] = m
+        state[sl[s]] = S[:, :, :dv]
+        mstate[sl[s]] = torch.cat([S[:, :, dv], m[:, None]], 1)
     return out
 
 

@@ -249,7 +249,7 @@ def test_sink_attention_through_shuffled_pages(device, dtype, l):
     for cuts in ([T], [5, 1, 2, T - 8], [1] * T):
         cache = (torch.zeros((nblk + 3) * bs, G * d, dtype=dtype, device=device),
                  torch.zeros((nblk + 3) * bs, G * dv, dtype=dtype, device=device),
-                 torch.zeros(2, 1, 4, 5, device=device), torch.zeros(2, 1, device=device))
+                 torch.zeros(2, 1, 4, 4, device=device), torch.zeros(2, 1, 5, device=device))
         got, at = [], 0
         for n in cuts:
             step = StepView(i32([0, n], device), n, i32(np.arange(at, at + n), device),
@@ -291,8 +291,8 @@ def test_recurrences_and_their_state(device, dtype, form, H_, d, dv):
     else:
         cache = (torch.zeros(3 * bs, 4, dtype=dtype, device=device),
                  torch.zeros(3 * bs, 4, dtype=dtype, device=device),
-                 torch.full((3, H_, d, dv + 1), 3.0, device=device),
-                 torch.full((3, H_), -2.0, device=device))
+                 torch.full((3, H_, d, dv), 3.0, device=device),
+                 torch.full((3, H_, d + 1), -2.0, device=device))
 
     def run(parts):             # parts: [(name, slot, start, n)]
         rows = np.concatenate([hs[nm][s:s + n] for nm, _, s, n in parts])
@@ -321,6 +321,45 @@ def test_recurrences_and_their_state(device, dtype, form, H_, d, dv):
     np.testing.assert_allclose(got, want["a"][22:], atol=a, rtol=a)
     st = cache[0] if form == "lightning" else cache[2]
     assert float(st[1].min()) == 3.0 and float(st[1].max()) == 3.0
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("form", ["lightning", "mlstm"])
+def test_long_portions_of_wide_states(device, dtype, form):
+    """Portions long enough, and states wide enough, that a head's state columns are dealt to
+    several workgroups (the matrix memory's norm then runs as a kernel of its own): a long
+    portion, single tokens, another portion, against the oracle over the whole sequence."""
+    from distributed_llm_inferencing_amd.models.mixers import (StepView, lightning_mixer,
+                                                               parallel_mixer)
+    D, eps, T, H_, d, dv = 32, 1e-5, 110, 2, 128, 128
+    if form == "lightning":
+        lay = lightning(H_, d, dv, decay=[0.97, 0.6])
+    else:
+        lay = parallel(l=left(heads=1, kv_heads=1, dim=4, vdim=4), r=right(H_, d, dv, cap=6.0),
+                       ls=0.0, rs=0.9)
+    c = config([lay], width=D)
+    w = O.random_weights(c, 3)
+    spec, lp = layer_params(c, w, device, dtype)
+    h = hidden(T, D, 5)
+    want = (O.lightning(h, w, "l0.mix.", lay["mixer"], eps) if form == "lightning"
+            else 0.9 * O.mlstm(h, w, "l0.mix.right.", lay["mixer"]["right"], eps))
+    bs = 128
+    cache = ((torch.full((2, H_, d, dv), 3.0, device=device),) if form == "lightning" else
+             (torch.zeros(2 * bs, 4, dtype=dtype, device=device),
+              torch.zeros(2 * bs, 4, dtype=dtype, device=device),
+              torch.full((2, H_, d, dv), 3.0, device=device),
+              torch.full((2, H_, d + 1), -2.0, device=device)))
+    got, at = [], 0
+    for n in (70, 1, 1, 38):
+        step = StepView(i32([0, n], device), n, i32(np.arange(at, at + n), device),
+                        i32(bs + np.arange(at, at + n), device), i32([[1]], device), bs,
+                        i32([1], device), at + n)
+        fn = lightning_mixer if form == "lightning" else parallel_mixer
+        got.append(fn(spec, lp, dev_t(h[at:at + n], device, dtype), step, cache,
+                      eps).float().cpu().numpy())
+        at += n
+    a = 3e-4 if dtype == torch.float32 else 6e-2
+    np.testing.assert_allclose(np.concatenate(got), want, atol=a, rtol=a)
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
