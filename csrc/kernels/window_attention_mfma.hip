@@ -76,6 +76,9 @@ struct MfmaArgs {
   // from (sink, 1) instead of (-inf, 0). head_gate: the gate row holds one number per head.
   // out_scale multiplies the output.
   const float* sink; int head_gate; float out_scale;
+  // value slice of a workgroup: 128 with all heads in it; in the wide form the whole value
+  // width up to 512 (narrower values take a narrower LDS image, so more workgroups share a CU)
+  int dvw;
   float* stats_ws;   // [S][q tiles][nsplit][H][TQ][2]
   float* o_ws;       // [nsplit][T][H*dv]
   long o_ws_stride;  // T * H * dv
@@ -99,7 +102,7 @@ __global__ void __launch_bounds__(512) window_attention_mfma_kernel(MfmaArgs a) 
   constexpr bool wide = WIDE;
   // 16-byte staging loads in flight per thread: what the register budget of the form allows
   constexpr int STG = WIDE ? 5 : 2;
-  const int dvw = wide ? 512 : 128;               // value slice of a workgroup
+  const int dvw = a.dvw;                          // value slice of a workgroup
   const int dvo = (blockIdx.z % a.ndvs) * dvw;
   const int hbase = ((blockIdx.z / a.ndvs) % a.nhs) * NW;
   const int split = blockIdx.z / (a.ndvs * a.nhs);
@@ -683,7 +686,7 @@ extern "C" int dli_window_attention_mfma(
   if (H < 1 || (!wide && H > NW * MAXHW) || G < 1 || (vrows == 0 && H % G) || H % Gk || dq % 32 || dv % 16 ||
       !aligned || window < 1 || block_size < 1 || (talk != nullptr && Gk != G))
     return (int)hipErrorNotSupported;
-  const int dvw = wide ? 512 : 128;
+  const int dvw = wide ? (dv >= 512 ? 512 : ((dv + 15) & ~15)) : 128;
   const int Hp = (H + 31) & ~31, Hp16 = (H + 15) & ~15;
   const int ldk = dq + 16;
   // the whole window's cache rows in LDS when they take at most 16 KB
@@ -699,6 +702,12 @@ extern "C" int dli_window_attention_mfma(
   int CG = (int)((budget - fixed) / per_cg);
   CG = CG > (G > Gk ? G : Gk) ? (G > Gk ? G : Gk) : CG;
   CG = CG > NW ? NW : CG;
+  // a wide workgroup's 8 heads read at most this many key / value heads
+  if (wide && !rowhead) {
+    const int hk = H / Gk, hv = H / G;
+    const int need = (NW - 1) / (hk < hv ? hk : hv) + 2;
+    CG = CG > need ? need : CG;
+  }
   int cgv = (int)(CG * (per_cg / 2) / ((size_t)dvw * 40));   // value groups that fit the regions
   cgv = cgv > G ? G : cgv;
   const size_t sh = fixed + CG * per_cg;
@@ -725,7 +734,7 @@ extern "C" int dli_window_attention_mfma(
   MfmaArgs a{(const u16*)q, ldq, (const u16*)k, k_stride, (const u16*)v, v_stride, (u16*)out,
              ldo, gate, ldg, slopes, talk, cu, positions, block_tables, bt_stride, block_size,
              H, G, dq, dv, window, scale, Gk, chunk, Hp, CG, 0, 1, ndvs, wide ? 1 : 0, nhs, rowmul,
-             vrows, cgv, slot_cap, sink, head_gate, out_scale, nullptr, nullptr, 0};
+             vrows, cgv, slot_cap, sink, head_gate, out_scale, dvw, nullptr, nullptr, 0};
   if (nsplit == 1) {
     dim3 grid(qtiles, num_seqs, ndvs * nhs);
     WA_LAUNCH(grid);
