@@ -245,6 +245,25 @@ __global__ void __launch_bounds__(256) rmsnorm_cols_kernel(
   }
 }
 
+// The same for few, wide rows (a decode step): one workgroup per row instead of one wave.
+template <typename S>
+__global__ void __launch_bounds__(256) rmsnorm_cols_block_kernel(
+    S* __restrict__ out, const float* __restrict__ src, int lds, const S* __restrict__ w, int n,
+    float eps, const float* __restrict__ gate, int ldg, int groups, int ldo, float out_scale) {
+  __shared__ float red[16];
+  const int t = blockIdx.x / groups, go = (blockIdx.x % groups) * n;
+  const float* r = src + (long)t * lds + go;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < n; c += blockDim.x) { const float v = r[c]; s += v * v; }
+  s = block_sum(s, red);
+  const float rs = 1.f / sqrtf(s / (float)n + eps);
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
+    float v = r[c] * rs * ldf(w + go + c);
+    if (gate != nullptr) v *= 1.f / (1.f + expf(-gate[(long)t * ldg + go + c]));
+    stf(out + (long)t * ldo + go + c, v * out_scale);
+  }
+}
+
 // The rotation of element c of a rotated part `v` (length >= rot_dims): with `half` dimension
 // i < rot_dims/2 pairs with i + rot_dims/2, else pairs are (2i, 2i+1). The pair (u, v) at angle
 // a becomes (u cos a - v sin a, v cos a + u sin a); the angle position * frequency is formed in
@@ -482,6 +501,15 @@ extern "C" int dli_rmsnorm_cols(void* out, const float* src, int lds, const void
                                 float out_scale, int dt, hipStream_t st) {
   if (T <= 0) return 0;
   if (n < 1 || groups < 1) return (int)hipErrorInvalidValue;
+  if ((long)T * groups <= 512 && n >= 1024) {
+    DT_SWITCH(dt,
+              (rmsnorm_cols_block_kernel<u16><<<T * groups, 256, 0, st>>>(
+                  (u16*)out, src, lds, (const u16*)w, n, eps, gate, ldg, groups, ldo, out_scale)),
+              (rmsnorm_cols_block_kernel<float><<<T * groups, 256, 0, st>>>(
+                  (float*)out, src, lds, (const float*)w, n, eps, gate, ldg, groups, ldo,
+                  out_scale)));
+    DLI_RETURN_LAUNCH();
+  }
   const int nb = (int)(((long)T * groups + 3) / 4);
   const bool vec4 = n % 4 == 0 && lds % 4 == 0 && ldg % 4 == 0 && ldo % 4 == 0 &&
                     (((uintptr_t)out | (uintptr_t)src | (uintptr_t)w | (uintptr_t)gate) & 15) == 0;

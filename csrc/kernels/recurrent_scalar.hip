@@ -46,6 +46,8 @@ __device__ __forceinline__ float logsigmoid32(float x) {
   return x > 0.f ? -log1pf(expf(-x)) : x - log1pf(expf(x));
 }
 
+// tokens per chunk (32 was measured: the walk gains little, the matrix memory's per-chunk
+// products and scans, which grow with the square of the chunk, lose more)
 constexpr int TC = 16;
 
 struct ScalarRecArgs {
@@ -162,8 +164,14 @@ __global__ void __launch_bounds__(1024) scalar_recurrence_kernel(ScalarRecArgs a
         if (tt >= n || j > tt) continue;
         const float* q = qv + tt * d;
         const float* k = j < 0 ? nvec : kv + j * d;
+        // rows are d floats apart (a multiple of the bank count for the usual d): every
+        // thread starts its walk at another element, so a wave's reads fall into distinct banks
         float acc = 0.f;
-        for (int i = 0; i < d; ++i) acc += k[i] * q[i];
+        int ii = idx % d;
+        for (int i = 0; i < d; ++i) {
+          acc += k[ii] * q[ii];
+          ii = ii + 1 == d ? 0 : ii + 1;
+        }
         if (j < 0) n0q[tt] = acc; else kq[idx] = acc;
       }
     }

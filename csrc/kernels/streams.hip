@@ -25,9 +25,10 @@ template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p =
 
 constexpr int MAXS = 8;          // streams
 
-// One workgroup per token. VEC = 4: 16-byte accesses of the fp32 rows (dim % 4 == 0).
+// One workgroup per token (256 threads; 1024 for the few wide rows of a decode step, which
+// are bound by latency). VEC = 4: 16-byte accesses of the fp32 rows (dim % 4 == 0).
 template <typename S, int VEC>
-__global__ void __launch_bounds__(256) hyper_mix_kernel(
+__global__ void __launch_bounds__(1024) hyper_mix_kernel(
     float* __restrict__ xs, const float* __restrict__ y, int ldy, const float* __restrict__ prev,
     const float* __restrict__ read, const S* __restrict__ w, void* __restrict__ h, int ns,
     int dim, float eps, float w_offset) {
@@ -110,7 +111,7 @@ __global__ void __launch_bounds__(256) hyper_mix_kernel(
 
 // One workgroup per token. proj row (fp32): [H*d q | G*d k | G*dv v | ...].
 template <typename S>
-__global__ void __launch_bounds__(256) sink_prepare_kernel(
+__global__ void __launch_bounds__(1024) sink_prepare_kernel(
     const float* __restrict__ proj, int ldp, const S* __restrict__ qw, const S* __restrict__ kw,
     float eps, int H, int G, int d, int dv, int rot, const double* __restrict__ freq,
     float mscale, const int* __restrict__ positions, S* __restrict__ q_out,
@@ -179,9 +180,10 @@ extern "C" int dli_hyper_mix(float* xs, const float* y, int ldy, const float* pr
   if (sh > 60000) return (int)hipErrorInvalidValue;
   const bool v4 = dim % 4 == 0 && (uintptr_t)xs % 16 == 0 &&
                   (y == nullptr || ((uintptr_t)y % 16 == 0 && ldy % 4 == 0));
+  const int nt = (T <= 1024 && dim >= 2048) ? 1024 : 256;
 #define HM_LAUNCH(S, V)                                                                       \
-  hyper_mix_kernel<S, V><<<T, 256, sh, st>>>(xs, y, ldy, prev, read, (const S*)w, h, ns, dim, \
-                                             eps, w_offset)
+  hyper_mix_kernel<S, V><<<T, nt, sh, st>>>(xs, y, ldy, prev, read, (const S*)w, h, ns, dim,  \
+                                            eps, w_offset)
   if (v4) DT_SWITCH2(dt, HM_LAUNCH(u16, 4), HM_LAUNCH(float, 4));
   else DT_SWITCH2(dt, HM_LAUNCH(u16, 1), HM_LAUNCH(float, 1));
 #undef HM_LAUNCH
@@ -199,11 +201,12 @@ extern "C" int dli_sink_prepare(const float* proj, int ldp, const void* qw, cons
     return (int)hipErrorInvalidValue;
   const size_t sh = ((size_t)(H + G) * d + rot_dims + 16) * 4;
   if (sh > 60000) return (int)hipErrorInvalidValue;
+  const int nt = (T <= 1024 && (H + G) * d >= 2048) ? 1024 : 256;
   DT_SWITCH2(dt,
-             (sink_prepare_kernel<u16><<<T, 256, sh, st>>>(
+             (sink_prepare_kernel<u16><<<T, nt, sh, st>>>(
                  proj, ldp, (const u16*)qw, (const u16*)kw, eps, H, G, d, dv, rot_dims, freq,
                  mscale, positions, (u16*)q_out, (u16*)kcache, (u16*)vcache, slots)),
-             (sink_prepare_kernel<float><<<T, 256, sh, st>>>(
+             (sink_prepare_kernel<float><<<T, nt, sh, st>>>(
                  proj, ldp, (const float*)qw, (const float*)kw, eps, H, G, d, dv, rot_dims, freq,
                  mscale, positions, (float*)q_out, (float*)kcache, (float*)vcache, slots)));
   DLI_RETURN_LAUNCH();
