@@ -212,7 +212,7 @@ def run_design_lapunex(a):
     D, Fw, V, Hh, G, hd = a.design_width, a.design_ff, 32000, a.design_width // 128, 8, 128
     E, top = 8, 2
     moe = dict(ff_kind="moe", router="group_score", expert_act="clamp_swish", ff=Fw, experts=E,
-               top=top, router_groups=4, router_keep=2, router_scale=1.5, act_limit=7.0)
+               top=top, router_groups=4, router_keep=2, router_scale=2.5, act_limit=7.0)
 
     def lightning():
         decays = tuple(1.0 - 2.0 ** (-1.0 - 7.0 * h / max(1, Hh - 1)) for h in range(Hh))
@@ -221,12 +221,12 @@ def run_design_lapunex(a):
     def parallel():
         left = LayerSpec("sink_attention", heads=Hh, kv_heads=G, dim=hd, vdim=hd,
                          scale=hd ** -0.5, rot_dims=64, rot_base=10000.0, window=1 << 30,
-                         rot_scaling=(8.0, 4096.0, 32.0, 1.0))
+                         rot_scaling=(4.0, 8192.0, 16.0, 2.0))
         right = LayerSpec("mlstm", heads=Hh // 2, dim=hd, vdim=hd, gate_cap=15.0)
         return LayerSpec("parallel", heads=Hh, kv_heads=G, dim=hd, vdim=hd, left=left,
-                         right=right, left_scale=0.8, right_scale=0.5, **moe)
+                         right=right, left_scale=0.7, right_scale=0.6, **moe)
     hyb = hybrid_config("lapunex-bench", D, V, (lightning(), parallel(), lightning(), parallel()),
-                        arch="lapunex", max_position=1 << 15, norm_eps=1e-5, embed_scale=12.0,
+                        arch="lapunex", max_position=1 << 15, norm_eps=1e-6, embed_scale=8.0,
                         streams=3, norm_offset=1.0, loop_entry=False)
     mix = replace(get_config("mixtral-8x7b"), name="mixtral-bench", hidden_size=D, num_layers=4,
                   num_heads=Hh, num_kv_heads=G, head_dim=hd, intermediate_size=Fw, vocab_size=V,

@@ -61,7 +61,7 @@ def parallel(l=None, r=None, ls=0.7, rs=1.2, mlp=None):
                                           "left_scale": ls, "right_scale": rs}, "mlp": mlp}
 
 
-def config(layers, width=40, vocab=80, eps=2e-5, scale=3.0, streams=3, loop=None):
+def config(layers, width=40, vocab=80, eps=2e-5, scale=3.0, streams=2, loop=None):
     c = {"architecture": "Lapunex", "width": width, "vocab": vocab, "norm": {"eps": eps},
          "embedding": {"scale": scale}, "layers": layers}
     if streams:
@@ -83,7 +83,7 @@ FULL = config([lightning(mlp=dense()), parallel(mlp=moe()),
                lightning(heads=3, dim=4, vdim=4, mlp=moe(experts=4, top=1, groups=(2, 1))),
                parallel(l=left(heads=2, kv_heads=2, dim=16, vdim=4, rot_=rot(16, 10.0, None)),
                         r=right(heads=1, dim=16, vdim=8, cap=3.0), mlp=None),
-               lightning(heads=1, dim=16, vdim=8, mlp=dense(24))], loop=(1, 4, 2))
+               lightning(heads=1, dim=16, vdim=8, mlp=dense(24))], streams=4, loop=(1, 3, 3))
 
 
 def engine(c, w, device, dtype, max_tokens=512, live=4, block_size=8, **kw):
@@ -206,7 +206,7 @@ def test_stream_mix_read_and_norm(device, dtype, S, D):
 
 def test_yarn_frequencies_follow_their_definition():
     from distributed_llm_inferencing_amd.models.mixers import yarn_frequencies
-    for r in (rot(), rot(16, 10000.0, (8.0, 512, 32.0, 1.0)), rot(6, 7.0, None),
+    for r in (rot(), rot(16, 10000.0, (6.0, 1024, 24.0, 2.0)), rot(6, 7.0, None),
               rot(32, 500.0, (2.5, 100, 9.0, 2.0)), rot(2, 100.0, (40.0, 4096, 1.0, 1.0))):
         sc = r.get("scaling")
         f, m = yarn_frequencies(r["dims"], r["base"],
@@ -215,9 +215,9 @@ def test_yarn_frequencies_follow_their_definition():
         np.testing.assert_allclose(f.numpy(), fo, rtol=1e-12)
         assert abs(m - mo) < 1e-12
     # a pair that turns often keeps its frequency, a slow one is divided by the factor
-    f, _ = yarn_frequencies(16, 10000.0, (8.0, 512.0, 32.0, 1.0))
+    f, _ = yarn_frequencies(16, 10000.0, (6.0, 1024.0, 24.0, 2.0))
     plain = 10000.0 ** (-2.0 * np.arange(8) / 16)
-    assert f[0] == plain[0] and abs(float(f[-1]) - plain[-1] / 8.0) < 1e-15
+    assert f[0] == plain[0] and abs(float(f[-1]) - plain[-1] / 6.0) < 1e-15
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
@@ -364,10 +364,10 @@ def test_long_portions_of_wide_states(device, dtype, form):
 
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("mlp", [moe(), moe(top=1), moe(experts=3, top=3, groups=(1, 1)),
-                                 moe(groups=None), moe(experts=8, top=4, groups=(4, 3)),
+                                 moe(groups=None), moe(experts=10, top=3, groups=(5, 3)),
                                  moe(ff=7, experts=9, top=3, groups=(3, 1), scale=0.4, limit=0.3),
                                  moe(experts=6, top=2, groups=(6, 2))],
-                         ids=["usual", "top1", "all_experts", "no_groups", "four_groups",
+                         ids=["usual", "top1", "all_experts", "no_groups", "five_groups",
                               "one_group_kept", "groups_of_one"])
 def test_router_and_experts(device, dtype, mlp):
     """Softmax scores, group-limited choice, scaled un-renormalised weights, clamped experts."""
@@ -418,7 +418,7 @@ def test_layer_trace_matches_the_oracle(device, dtype):
     eng = engine(FULL, w, device, dtype)
     eng.model.layer_trace = []
     replay(eng, t, [14])
-    assert len(eng.model.layer_trace) == len(trace) == 8          # 1 + 3 * 2 + 1 runs
+    assert len(eng.model.layer_trace) == len(trace) == 9          # 1 + 2 * 3 + 2 runs
     for i, (got, want) in enumerate(zip(eng.model.layer_trace, trace)):
         d = np.abs(got.cpu().numpy() - want).max(-1)
         lim = 1e-3 if dtype == torch.float32 else 3e-2 * np.abs(want).max()
@@ -599,8 +599,8 @@ def test_config_reader_reads_every_size():
     cfg = config_from_hf(FULL)
     assert cfg.arch == "lapunex" and cfg.is_hybrid and cfg.has_state
     assert (cfg.hidden_size, cfg.vocab_size, cfg.embed_scale, cfg.norm_eps) == (40, 80, 3.0, 2e-5)
-    assert cfg.streams == 3 and cfg.loop == (1, 4, 2) and not cfg.loop_entry
-    assert [li for li, _, first in cfg.layer_runs() if not first] == [0, 1, 2, 3, 1, 2, 3, 4]
+    assert cfg.streams == 4 and cfg.loop == (1, 3, 3) and not cfg.loop_entry
+    assert [li for li, _, first in cfg.layer_runs() if not first] == [0, 1, 2, 1, 2, 1, 2, 3, 4]
     s = cfg.layer_specs
     assert [x.kind for x in s] == ["lightning", "parallel", "lightning", "parallel", "lightning"]
     assert (s[0].heads, s[0].dim, s[0].vdim, s[0].ff_kind, s[0].ff) == (2, 8, 12, "gated_silu", 40)
@@ -618,7 +618,7 @@ def test_config_reader_reads_every_size():
     assert ModelConfig.from_dict(cfg.to_dict()) == cfg
     params = from_lapunex_state_dict(cfg, {k: torch.as_tensor(v) for k, v in
                                            O.random_weights(FULL, 0).items()})
-    assert params["layers.1.hc2"].shape == (15,) and params["layers.1.hc2"].dtype == torch.float32
+    assert params["layers.1.hc2"].shape == (24,) and params["layers.1.hc2"].dtype == torch.float32
     assert params["layers.1.wo"].shape == (40, 4 * 6 + 2 * 10)
     bad = copy.deepcopy(FULL)
     bad["layers"][1]["mlp"]["router"]["groups"]["count"] = 4      # 6 experts in 4 groups
