@@ -283,9 +283,11 @@ def random_weights(c, seed=0):
                 continue
             w[f"{a}norm{q}"] = rng.standard_normal(D) * 0.2
             if ns:
-                w[f"{a}hc{q}.in"] = 1.0 / ns + 0.2 * rng.standard_normal(ns)
+                # read weights that do not cancel: a sum of streams much smaller than the
+                # streams would magnify every rounding in front of the norm
+                w[f"{a}hc{q}.in"] = (1.0 + 0.3 * rng.standard_normal(ns)) / ns
                 w[f"{a}hc{q}.out"] = 1.0 + 0.3 * rng.standard_normal(ns)
-                w[f"{a}hc{q}.mix"] = np.eye(ns) + 0.2 * rng.standard_normal((ns, ns))
+                w[f"{a}hc{q}.mix"] = np.eye(ns) + 0.15 * rng.standard_normal((ns, ns))
         m = a + "mix."
         if L["type"] == "lightning":
             H, d, dv = int(mx["heads"]), int(mx["dim"]), int(mx["vdim"])

@@ -122,7 +122,7 @@ def close(got, want, dtype, what="", slack=1.0):
     loose = None
     if isinstance(want, Ref):
         if dtype == torch.bfloat16:
-            loose = np.maximum.accumulate(want.margins < 0.02)
+            loose = np.maximum.accumulate(want.margins < 0.03)
         want = want.logits
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     d = got - want
@@ -439,9 +439,11 @@ def test_prefill_equals_decode_equals_portions(device, dtype, routed):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-def test_mixed_batches_and_reuse_of_pages_and_slots(device, dtype):
+@pytest.mark.parametrize("routed", [True, False])
+def test_mixed_batches_and_reuse_of_pages_and_slots(device, dtype, routed):
     """Unequal requests in one step (portions beside single tokens) against each alone, in a
     pool so small that pages and state slots are freed and taken again."""
+    FULL = globals()["FULL"] if routed else without_routing(globals()["FULL"])
     w = O.random_weights(FULL, 4)
     V = FULL["vocab"]
     seqs = {k: toks(n, V, s) for k, n, s in (("a", 30, 1), ("b", 9, 2), ("c", 17, 3), ("d", 5, 4),
