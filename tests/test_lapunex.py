@@ -664,3 +664,39 @@ def test_tuned_layouts_and_matrix_core_attention(width, lay, n):
     close(replay(eng, t, [n]), want, torch.bfloat16, "whole")
     close(replay(eng, t, [n - 9, 2, 1, 1, 5]), want, torch.bfloat16, "portions")
     close(replay(eng, t, [n - 20] + [1] * 20), want, torch.bfloat16, "decoded")
+
+
+def test_checkpoint_folder_through_the_replay_command(tmp_path, monkeypatch, capsys):
+    """A checkpoint folder (config.json + model.safetensors in bfloat16) read by the C++
+    safetensors loader, and the trace replay command driving the engine: two requests in mixed
+    steps, logits written per step."""
+    import io
+    import json
+    from safetensors.torch import save_file
+    from distributed_llm_inferencing_amd.cli import main as cli_main
+    c = config([lightning(mlp=moe()), parallel(mlp=dense())], loop=(0, 2, 2))
+    w = O.random_weights(c, 21)
+    model = tmp_path / "model"
+    model.mkdir()
+    (model / "config.json").write_text(json.dumps(c))
+    save_file({k: torch.as_tensor(v).to(torch.bfloat16).contiguous() for k, v in w.items()},
+              str(model / "model.safetensors"))
+    ta, tb = toks(21, c["vocab"], 1), toks(9, c["vocab"], 2)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": ta[:13], "want": [0, 12]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": ta[13:14], "want": [0]},
+                                     {"id": "b", "tokens": tb, "want": [3, 8]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": ta[14:], "want": []}], "end": ["a"]}]
+    monkeypatch.setattr("sys.stdin", io.StringIO("\n".join(json.dumps(s) for s in steps) + "\n"))
+    out = tmp_path / "out"
+    rc = cli_main(["trace-run", "--model", str(model), "--dtype", "float32", "--out", str(out),
+                   "--max-tokens", "128", "--device", "cpu"])
+    assert rc == 0
+    assert [ln for ln in capsys.readouterr().out.splitlines() if ln.startswith("done")] == \
+        ["done 0", "done 1", "done 2"]
+    ra, rb = O.forward(c, w, ta), O.forward(c, w, tb)
+    V = c["vocab"]
+    got0 = np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V)
+    got1 = np.fromfile(out / "1.f32", dtype="<f4").reshape(-1, V)
+    close(got0, ra[[0, 12]], torch.float32, "step 0")
+    close(got1, np.stack([ra[13], rb[3], rb[8]]), torch.float32, "step 1")
+    assert not (out / "2.f32").exists()
