@@ -121,18 +121,20 @@ __global__ void __launch_bounds__(1024) scalar_recurrence_kernel(ScalarRecArgs a
   for (int tc = t0; tc < t1; tc += TC) {
     const int n = min(TC, t1 - tc);
     __syncthreads();                           // the previous chunk is done with the LDS rows
-    for (int i = threadIdx.x; i < n * dvp; i += blockDim.x) {
-      const int tt = i / dvp, cc = i % dvp;
+    // (thread = (row group `part`, column c): token part + u P, column c — no divisions; with
+    // the rows in registers d is the constant D, a power of two)
+    for (int tt = part; tt < n; tt += P) {
       float v = 0.f;
-      if (cc < ncol) {
-        v = a.proj[(long)(tc + tt) * a.ldp + voff + cc];
+      if (c < ncol) {
+        v = a.proj[(long)(tc + tt) * a.ldp + voff + c];
         if (FORM == 0) v = silu32(v);
       }
-      vv[i] = v;
+      vv[tt * dvp + c] = v;
     }
-    for (int i = threadIdx.x; i < n * d; i += blockDim.x) {
-      const float* row = a.proj + (long)(tc + i / d) * a.ldp + h * d + i % d;
-      const float q = row[0], k = row[H * d];
+    const int dd = D ? D : d;
+    for (int i = threadIdx.x; i < n * dd; i += blockDim.x) {
+      const float* row = a.proj + (long)(tc + i / dd) * a.ldp + h * dd + i % dd;
+      const float q = row[0], k = row[H * dd];
       qv[i] = FORM == 0 ? silu32(q) : q * qscale;
       kv[i] = FORM == 0 ? silu32(k) : k;
     }
@@ -162,15 +164,15 @@ __global__ void __launch_bounds__(1024) scalar_recurrence_kernel(ScalarRecArgs a
         const int tt = idx < TC * TC ? idx / TC : idx - TC * TC;
         const int j = idx < TC * TC ? idx % TC : -1;
         if (tt >= n || j > tt) continue;
-        const float* q = qv + tt * d;
-        const float* k = j < 0 ? nvec : kv + j * d;
+        const float* q = qv + tt * dd;
+        const float* k = j < 0 ? nvec : kv + j * dd;
         // rows are d floats apart (a multiple of the bank count for the usual d): every
         // thread starts its walk at another element, so a wave's reads fall into distinct banks
         float acc = 0.f;
-        int ii = idx % d;
-        for (int i = 0; i < d; ++i) {
+        int ii = idx % dd;
+        for (int i = 0; i < dd; ++i) {
           acc += k[ii] * q[ii];
-          ii = ii + 1 == d ? 0 : ii + 1;
+          ii = ii + 1 == dd ? 0 : ii + 1;
         }
         if (j < 0) n0q[tt] = acc; else kq[idx] = acc;
       }

@@ -69,7 +69,9 @@ class HybridLM(TransformerLM):
             derive_constants(spec, lp, self.device)
         self._cu: Dict[int, torch.Tensor] = {}
         self._rows: Dict[int, torch.Tensor] = {}
-        self._sum_streams: Optional[torch.Tensor] = None
+        # read weights of the plain sum of the streams (made here, not inside a captured step)
+        self._sum_streams = (torch.ones(cfg.streams, dtype=torch.float32, device=self.device)
+                             if cfg.streams else None)
         # debugging aid: when a list, forward_layers appends the residual after every run
         self.layer_trace: Optional[List[torch.Tensor]] = None
 
@@ -82,6 +84,9 @@ class HybridLM(TransformerLM):
             derive_constants(spec, lp, self.device)
         self._cu.clear()
         self._rows.clear()
+        if self.cfg.streams:
+            self._sum_streams = torch.ones(self.cfg.streams, dtype=torch.float32,
+                                           device=self.device)
         return self
 
     # ------------------------------------------------------------------ step metadata
@@ -151,8 +156,6 @@ class HybridLM(TransformerLM):
         step = self._step_view(b, kv_caches.block_size)
         T, D = x.shape
         xs = x.unsqueeze(1).expand(T, S, D).contiguous()
-        if self._sum_streams is None or self._sum_streams.device != x.device:
-            self._sum_streams = torch.ones(S, dtype=torch.float32, device=x.device)
         y = prev = None                     # a sublayer's output awaiting its write-back
         for ri, (li, _, _) in enumerate(self.runs):
             spec, lp = cfg.layer_specs[li], self.layers[li]
