@@ -641,15 +641,20 @@ def lightning(proj, decays, state, slots, cu_seqlens, max_seqlen, positions, H, 
     out = torch.empty(T, H * dv, dtype=torch.float32, device=proj.device)
     _call("dli_scalar_recurrence", _p(proj), proj.stride(0), 0, _p(decays), None, 0.0, None, 0.0,
           _p(state), None, _p(slots), _p(cu_seqlens), _p(positions), _p(out), out.stride(0), 1.0,
-          S, int(max_seqlen), H, d, dv, _column_block(S, H, dv, max_seqlen), None, 1, _st())
+          S, int(max_seqlen), H, d, dv, _column_block(S, H, d, dv, max_seqlen), None, 1, _st())
     return out
 
 
-def _column_block(S: int, H: int, dv: int, max_seqlen: int) -> int:
+def _column_block(S: int, H: int, d: int, dv: int, max_seqlen: int) -> int:
     """State columns per workgroup of a recurrence over a step's portions: few (head,
     sequence) pairs with long portions leave most of the chip idle, so the columns are dealt
-    to several workgroups (0: one workgroup holds all of them)."""
-    return 64 if (S * H < 256 and max_seqlen >= 64 and dv >= 128) else 0
+    to several workgroups (0: one workgroup holds all of them). States too wide for one
+    workgroup's registers (d in 16 / 32 / 64 / 128) or LDS (any other d) are always dealt."""
+    if S * H < 256 and max_seqlen >= 64 and dv >= 128:
+        return 64
+    if d in (16, 32, 64, 128):
+        return 256 if dv > 256 else 0
+    return 64 if dv > 64 and d * ((dv + 63) // 64 * 64) * 4 > 96 * 1024 else 0
 
 
 def mlstm(proj, if_b, cap: float, norm_w, eps: float, state, mstate, slots, cu_seqlens,
@@ -662,7 +667,7 @@ def mlstm(proj, if_b, cap: float, norm_w, eps: float, state, mstate, slots, cu_s
         return R.mlstm(proj, if_b, cap, norm_w, eps, state, mstate, slots, cu_seqlens, positions,
                        H, d, dv, out, out_scale)
     S = cu_seqlens.shape[0] - 1
-    cw = _column_block(S, H, dv, max_seqlen)
+    cw = _column_block(S, H, d, dv, max_seqlen)
     # with column blocks no workgroup sees a whole head: the read-outs leave in fp32 and the
     # per-head norm, gate and scale run as a row kernel
     raw = torch.empty(proj.shape[0], H * dv, dtype=torch.float32, device=proj.device) if cw else None

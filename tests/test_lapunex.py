@@ -510,6 +510,26 @@ def test_other_sizes_and_degenerate_values(device, dtype):
         close(replay(eng, t, [3, 1, 2, 13]), want, dtype, f"config {n} portions")
 
 
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_states_wider_than_a_workgroup(device, dtype):
+    """States whose columns exceed what one workgroup keeps in registers (d a power of two) or
+    in LDS (any other d): the columns are dealt to several workgroups in every step kind."""
+    att = left(heads=2, kv_heads=1, dim=32, vdim=16, rot_=rot(8))
+    cs = [config([lightning(heads=1, dim=128, vdim=320, mlp=None),
+                  parallel(l=att, r=right(heads=1, dim=128, vdim=384), mlp=dense(64))],
+                 width=64, vocab=90),
+          config([lightning(heads=1, dim=200, vdim=192, mlp=None),
+                  parallel(l=att, r=right(heads=1, dim=200, vdim=192), mlp=None)],
+                 width=64, vocab=90, streams=0)]
+    for n, c in enumerate(cs):
+        w = O.random_weights(c, 3)
+        t = toks(24, c["vocab"], 2)
+        want = ref(t, c, w)
+        eng = engine(c, w, device, dtype, max_tokens=128)
+        close(replay(eng, t, [24]), want, dtype, f"config {n} whole")
+        close(replay(eng, t, [17] + [1] * 7), want, dtype, f"config {n} decoded")
+
+
 def standout_model():
     """One parallel layer whose attention finds one key: keys and queries share their
     projection and norm weights (one key head per query head), so among unit-RMS rows a key
